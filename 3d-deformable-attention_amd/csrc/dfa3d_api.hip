@@ -1,0 +1,185 @@
+// C ABI of libdfa3d_hip (declared in include/dfa3d.h): argument checks and dispatch.
+// Errors are returned, never printed-and-ignored (the reference's launchers only printf a failed
+// launch: DFA3D/dfa3D/ops/csrc/cuda/wms_deform_attn_cuda.cu:45-48).
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "../../include/dfa3d.h"
+#include "dfa3d_launch.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_result(hipError_t e, const char *what) {
+  if (e == hipSuccess) return 0;
+  return fail((int)e, "%s: %s", what, hipGetErrorString(e));
+}
+
+// Process-wide launch tunables (dfa3d_set_tunable); initial values may come from the environment
+// variables DFA3D_ITERS / DFA3D_VEC.
+int env_int(const char *name, int dflt) {
+  const char *s = getenv(name);
+  return (s && *s) ? atoi(s) : dflt;
+}
+std::atomic<int> g_iters{env_int("DFA3D_ITERS", 1)};
+std::atomic<int> g_vec{env_int("DFA3D_VEC", 0)};
+int tune_iters() { const int v = g_iters.load(std::memory_order_relaxed); return v < 1 ? 1 : v; }
+int tune_vec() { return g_vec.load(std::memory_order_relaxed); }
+
+// Dimension checks shared by every entry point.  `width` is the per-head row length (C or D).
+int check_dims(const char *fn, int B, int S, int M, int width, int L, int Q, int P, int dtype) {
+  if (dtype != DFA3D_F32 && dtype != DFA3D_F64 && dtype != DFA3D_BF16)
+    return fail(DFA3D_EINVAL, "%s: unknown dtype %d", fn, dtype);
+  if (B <= 0 || S <= 0 || M <= 0 || width <= 0 || L <= 0 || Q <= 0 || P <= 0)
+    return fail(DFA3D_EINVAL, "%s: dimensions must be positive (B=%d S=%d M=%d C|D=%d L=%d Q=%d P=%d)", fn, B, S, M,
+                width, L, Q, P);
+  if (L > DFA3D_MAX_LEVELS) return fail(DFA3D_ERANGE, "%s: L=%d exceeds %d levels", fn, L, DFA3D_MAX_LEVELS);
+  // one batch element of value / dist and of their gradients is addressed with 32-bit byte
+  // offsets that must stay below 2^30 (see kMaxSliceBytes)
+  const long long slice = (long long)S * M * width * (dtype == DFA3D_F64 ? 8 : 4);
+  if (slice >= (1LL << 30))
+    return fail(DFA3D_ERANGE, "%s: one batch element of a (B,S,M,%d) tensor takes %lld bytes, limit is 2^30", fn,
+                width, slice);
+  if ((long long)L * P > (1 << 20)) return fail(DFA3D_ERANGE, "%s: L*P=%lld too large", fn, (long long)L * P);
+  if ((long long)B * Q * M >= (1LL << 40)) return fail(DFA3D_ERANGE, "%s: B*Q*M too large", fn);
+  return 0;
+}
+
+#define REQUIRE_PTR(fn, p) \
+  if ((p) == nullptr) return fail(DFA3D_EINVAL, "%s: %s is NULL", fn, #p)
+
+}  // namespace
+
+extern "C" {
+
+const char *dfa3d_last_error(void) { return g_err; }
+int dfa3d_abi_version(void) { return 1; }
+
+int dfa3d_set_tunable(const char *name, int value) {
+  if (name == nullptr) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: name is NULL");
+  if (!strcmp(name, "iters")) {
+    if (value < 1 || value > 64) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: iters must be in [1, 64]");
+    g_iters.store(value, std::memory_order_relaxed);
+    return 0;
+  }
+  if (!strcmp(name, "vec")) {
+    if (value != 0 && value != 1 && value != 2 && value != 4)
+      return fail(DFA3D_EINVAL, "dfa3d_set_tunable: vec must be 0 (automatic), 1, 2 or 4");
+    g_vec.store(value, std::memory_order_relaxed);
+    return 0;
+  }
+  return fail(DFA3D_EINVAL, "dfa3d_set_tunable: unknown tunable '%s'", name);
+}
+
+int dfa3d_ms_depth_score_sample_forward(const void *dist, const int64_t *shapes3, const int64_t *level_start,
+                                        const void *loc3, void *score, int B, int S, int M, int D, int L, int Q, int P,
+                                        int dtype, void *stream) {
+  const char *fn = "dfa3d_ms_depth_score_sample_forward";
+  if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
+  REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, score);
+  dfa3d::DepthScoreArgs a{dist, shapes3, level_start, loc3, score, B, S, M, D, L, Q, P};
+  return hip_result(dfa3d::launch_depth_score(a, dtype, (hipStream_t)stream), fn);
+}
+
+int dfa3d_ms_depth_score_sample_backward(const void *dist, const int64_t *shapes3, const int64_t *level_start,
+                                         const void *loc3, const void *grad_score, void *grad_dist, void *grad_loc3,
+                                         int B, int S, int M, int D, int L, int Q, int P, int dtype, void *stream) {
+  const char *fn = "dfa3d_ms_depth_score_sample_backward";
+  if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start); REQUIRE_PTR(fn, loc3);
+  REQUIRE_PTR(fn, grad_score); REQUIRE_PTR(fn, grad_dist); REQUIRE_PTR(fn, grad_loc3);
+  dfa3d::DepthScoreBwdArgs a{dist, shapes3, level_start, loc3, grad_score, grad_dist, grad_loc3, B, S, M, D, L, Q, P};
+  return hip_result(dfa3d::launch_depth_score_backward(a, dtype, (hipStream_t)stream), fn);
+}
+
+int dfa3d_wms_deform_attn_forward(const void *value, const int64_t *shapes, int shape_stride,
+                                  const int64_t *level_start, const void *loc, int loc_stride, const void *attn,
+                                  const void *score, void *out, int B, int S, int M, int C, int L, int Q, int P,
+                                  int dtype, void *stream) {
+  const char *fn = "dfa3d_wms_deform_attn_forward";
+  if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
+  if (shape_stride < 2 || shape_stride > 3 || loc_stride < 2 || loc_stride > 3)
+    return fail(DFA3D_EINVAL, "%s: shape_stride and loc_stride must be 2 or 3", fn);
+  REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, shapes); REQUIRE_PTR(fn, level_start); REQUIRE_PTR(fn, loc);
+  REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, score); REQUIRE_PTR(fn, out);
+  dfa3d::FwdArgs a{};
+  a.value = value; a.dist = nullptr; a.shapes = shapes; a.shape_stride = shape_stride; a.level_start = level_start;
+  a.loc = loc; a.loc_stride = loc_stride; a.attn = attn; a.score_in = score; a.out = out; a.score_out = nullptr;
+  a.B = B; a.S = S; a.M = M; a.C = C; a.D = 1; a.L = L; a.Q = Q; a.P = P;
+  a.iters = tune_iters(); a.vec_hint = tune_vec();
+  return hip_result(dfa3d::launch_forward(a, dtype, (hipStream_t)stream), fn);
+}
+
+int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int shape_stride,
+                                   const int64_t *level_start, const void *loc, int loc_stride, const void *attn,
+                                   const void *score, const void *grad_out, void *grad_value, void *grad_loc,
+                                   int grad_loc_stride, void *grad_attn, void *grad_score, int B, int S, int M, int C,
+                                   int L, int Q, int P, int dtype, void *stream) {
+  const char *fn = "dfa3d_wms_deform_attn_backward";
+  if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
+  if (shape_stride < 2 || shape_stride > 3 || loc_stride < 2 || loc_stride > 3 || grad_loc_stride < 2 ||
+      grad_loc_stride > 3)
+    return fail(DFA3D_EINVAL, "%s: shape_stride, loc_stride and grad_loc_stride must be 2 or 3", fn);
+  REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, shapes); REQUIRE_PTR(fn, level_start); REQUIRE_PTR(fn, loc);
+  REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, score); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
+  REQUIRE_PTR(fn, grad_loc); REQUIRE_PTR(fn, grad_attn); REQUIRE_PTR(fn, grad_score);
+  dfa3d::BwdArgs a{};
+  a.value = value; a.dist = nullptr; a.shapes = shapes; a.shape_stride = shape_stride; a.level_start = level_start;
+  a.loc = loc; a.loc_stride = loc_stride; a.attn = attn; a.score_in = score; a.grad_out = grad_out;
+  a.grad_score_in = nullptr; a.grad_value = grad_value; a.grad_dist = nullptr; a.grad_loc = grad_loc;
+  a.grad_loc_stride = grad_loc_stride; a.grad_attn = grad_attn; a.grad_score_out = grad_score;
+  a.B = B; a.S = S; a.M = M; a.C = C; a.D = 1; a.L = L; a.Q = Q; a.P = P;
+  a.iters = tune_iters(); a.vec_hint = tune_vec();
+  return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
+}
+
+int dfa3d_fused_forward(const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
+                        const void *loc3, const void *attn, void *out, void *score, int B, int S, int M, int C, int D,
+                        int L, int Q, int P, int dtype, void *stream) {
+  const char *fn = "dfa3d_fused_forward";
+  if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
+  if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
+  REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, out);
+  dfa3d::FwdArgs a{};
+  a.value = value; a.dist = dist; a.shapes = shapes3; a.shape_stride = 3; a.level_start = level_start;
+  a.loc = loc3; a.loc_stride = 3; a.attn = attn; a.score_in = nullptr; a.out = out; a.score_out = score;
+  a.B = B; a.S = S; a.M = M; a.C = C; a.D = D; a.L = L; a.Q = Q; a.P = P;
+  a.iters = tune_iters(); a.vec_hint = tune_vec();
+  return hip_result(dfa3d::launch_forward(a, dtype, (hipStream_t)stream), fn);
+}
+
+int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
+                         const void *loc3, const void *attn, const void *grad_out, const void *grad_score_in,
+                         void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn, int B, int S, int M,
+                         int C, int D, int L, int Q, int P, int dtype, void *stream) {
+  const char *fn = "dfa3d_fused_backward";
+  if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
+  if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
+  REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
+  REQUIRE_PTR(fn, grad_dist); REQUIRE_PTR(fn, grad_loc3); REQUIRE_PTR(fn, grad_attn);
+  dfa3d::BwdArgs a{};
+  a.value = value; a.dist = dist; a.shapes = shapes3; a.shape_stride = 3; a.level_start = level_start;
+  a.loc = loc3; a.loc_stride = 3; a.attn = attn; a.score_in = nullptr; a.grad_out = grad_out;
+  a.grad_score_in = grad_score_in; a.grad_value = grad_value; a.grad_dist = grad_dist; a.grad_loc = grad_loc3;
+  a.grad_loc_stride = 3; a.grad_attn = grad_attn; a.grad_score_out = nullptr;
+  a.B = B; a.S = S; a.M = M; a.C = C; a.D = D; a.L = L; a.Q = Q; a.P = P;
+  a.iters = tune_iters(); a.vec_hint = tune_vec();
+  return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
+}
+
+}  // extern "C"

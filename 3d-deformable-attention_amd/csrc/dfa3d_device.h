@@ -1,0 +1,324 @@
+// Device-side building blocks shared by the forward and backward kernels of the DFA3D
+// operator on gfx950 (wave64).
+//
+// Work decomposition used by every kernel in this library:
+//   * a "unit" is one (batch b, query q, head m): L*P sampling points that are contiguous
+//     in the location / attention / score tensors and all gather from head m of batch b;
+//   * phase A ("lanes over points"): each lane of a wavefront owns one sampling point, does
+//     the index arithmetic, the depth-bin gathers and the coalesced reads/writes of the
+//     per-point tensors, and leaves one (row byte offset, weight) task per corner in LDS;
+//   * phase B ("lanes over channels"): the wavefront walks those tasks; LPR lanes of VEC
+//     channels each cover one value row, so one vector load instruction fetches 64/LPR rows,
+//     each fully coalesced.
+// The semantics (pixel coordinates, skip predicates, zero padding per corner and per depth
+// bin, corner slot order LT,RT,RB,LB) are those of the reference kernels
+//   DFA3D/dfa3D/ops/csrc/common/cuda/ms_depth_score_sample_cuda_kernel.cuh:24-148 and
+//   DFA3D/dfa3D/ops/csrc/common/cuda/wms_deform_attn_cuda_kernel.cuh:24-80,240-303.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#include "../../include/dfa3d.h"
+
+namespace dfa3d {
+
+constexpr int kWave = 64;
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = kWave * kWavesPerBlock;
+
+// ---------------------------------------------------------------------------------------
+// element access: storage type T -> arithmetic type A
+// ---------------------------------------------------------------------------------------
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+  static __device__ __forceinline__ float ld(const float *p) { return *p; }
+  static __device__ __forceinline__ void st(float *p, float v) { *p = v; }
+};
+template <> struct Elem<double> {
+  static __device__ __forceinline__ double ld(const double *p) { return *p; }
+  static __device__ __forceinline__ void st(double *p, double v) { *p = v; }
+};
+template <> struct Elem<__hip_bfloat16> {
+  static __device__ __forceinline__ float ld(const __hip_bfloat16 *p) {
+    return __uint_as_float(((uint32_t) * reinterpret_cast<const uint16_t *>(p)) << 16);
+  }
+  static __device__ __forceinline__ void st(__hip_bfloat16 *p, float v) { *p = __float2bfloat16(v); }
+};
+
+// ---------------------------------------------------------------------------------------
+// Buffer-addressed access.  One batch element of value / dist / grad_value / grad_dist is
+// described by a raw buffer resource (base, size in bytes); gathers and scatter-adds then take
+// a 32-bit byte offset, and an offset at or beyond the size reads as zero / drops the atomic in
+// hardware.  Tasks that have nothing to gather carry kNoRow as their offset, so phase B needs
+// no branches and can keep many gathers in flight; the same range check means no offset, however
+// wrong, can touch memory outside the tensor.
+// ---------------------------------------------------------------------------------------
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t kNoRow = 0x80000000u;    // offset of a task with nothing to gather
+constexpr uint32_t kNoChan = 0x40000000u;   // channel offset of a lane beyond the last channel
+// With every tensor slice below 2^30 bytes, kNoRow + x and row + kNoChan are out of range for
+// every in-range row offset and channel offset x (no 32-bit wrap-around).
+constexpr long long kMaxSliceBytes = 1LL << 30;
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, size_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __uint_as_float(b << 16); }
+
+// one element at byte offset `off`
+template <typename T> struct BufElem;
+template <> struct BufElem<float> {
+  static __device__ __forceinline__ float ld(rsrc_t r, uint32_t off) {
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
+  }
+};
+template <> struct BufElem<double> {
+  static __device__ __forceinline__ double ld(rsrc_t r, uint32_t off) {
+    const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+    return __hiloint2double((int)t.y, (int)t.x);
+  }
+};
+template <> struct BufElem<__hip_bfloat16> {
+  static __device__ __forceinline__ float ld(rsrc_t r, uint32_t off) {
+    return bf16_bits_to_float(__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0));
+  }
+};
+
+// VEC consecutive elements of a row at byte offset `off` (aligned to VEC elements)
+template <typename T, typename A, int VEC> struct RowVec;
+template <typename A> struct RowVec<float, A, 1> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[1]) { v[0] = BufElem<float>::ld(r, off); }
+  static __device__ __forceinline__ void st(float *p, const A (&v)[1]) { p[0] = v[0]; }
+};
+template <typename A> struct RowVec<float, A, 2> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[2]) {
+    const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+    v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y);
+  }
+  static __device__ __forceinline__ void st(float *p, const A (&v)[2]) {
+    *reinterpret_cast<float2 *>(p) = make_float2(v[0], v[1]);
+  }
+};
+template <typename A> struct RowVec<float, A, 4> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[4]) {
+    const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y);
+    v[2] = __uint_as_float(t.z); v[3] = __uint_as_float(t.w);
+  }
+  static __device__ __forceinline__ void st(float *p, const A (&v)[4]) {
+    *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <typename A> struct RowVec<double, A, 1> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[1]) { v[0] = BufElem<double>::ld(r, off); }
+  static __device__ __forceinline__ void st(double *p, const A (&v)[1]) { p[0] = v[0]; }
+};
+template <typename A> struct RowVec<double, A, 2> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[2]) {
+    const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    v[0] = __hiloint2double((int)t.y, (int)t.x); v[1] = __hiloint2double((int)t.w, (int)t.z);
+  }
+  static __device__ __forceinline__ void st(double *p, const A (&v)[2]) {
+    *reinterpret_cast<double2 *>(p) = make_double2(v[0], v[1]);
+  }
+};
+template <typename A> struct RowVec<double, A, 4> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[4]) {
+    const u32x4 t0 = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    const u32x4 t1 = __builtin_amdgcn_raw_buffer_load_b128(r, off + 16, 0, 0);
+    v[0] = __hiloint2double((int)t0.y, (int)t0.x); v[1] = __hiloint2double((int)t0.w, (int)t0.z);
+    v[2] = __hiloint2double((int)t1.y, (int)t1.x); v[3] = __hiloint2double((int)t1.w, (int)t1.z);
+  }
+  static __device__ __forceinline__ void st(double *p, const A (&v)[4]) {
+    reinterpret_cast<double2 *>(p)[0] = make_double2(v[0], v[1]);
+    reinterpret_cast<double2 *>(p)[1] = make_double2(v[2], v[3]);
+  }
+};
+template <typename A> struct RowVec<__hip_bfloat16, A, 1> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[1]) {
+    v[0] = BufElem<__hip_bfloat16>::ld(r, off);
+  }
+  static __device__ __forceinline__ void st(__hip_bfloat16 *p, const A (&v)[1]) { p[0] = __float2bfloat16(v[0]); }
+};
+template <typename A> struct RowVec<__hip_bfloat16, A, 2> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[2]) {
+    const uint32_t t = __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0);
+    v[0] = __uint_as_float(t << 16);
+    v[1] = __uint_as_float(t & 0xFFFF0000u);
+  }
+  static __device__ __forceinline__ void st(__hip_bfloat16 *p, const A (&v)[2]) {
+    p[0] = __float2bfloat16(v[0]);
+    p[1] = __float2bfloat16(v[1]);
+  }
+};
+template <typename A> struct RowVec<__hip_bfloat16, A, 4> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[4]) {
+    const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+    v[0] = __uint_as_float(t.x << 16);
+    v[1] = __uint_as_float(t.x & 0xFFFF0000u);
+    v[2] = __uint_as_float(t.y << 16);
+    v[3] = __uint_as_float(t.y & 0xFFFF0000u);
+  }
+  static __device__ __forceinline__ void st(__hip_bfloat16 *p, const A (&v)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) p[i] = __float2bfloat16(v[i]);
+  }
+};
+
+// Hardware floating-point scatter-add (no compare-and-swap loop) at byte offset `off` of a
+// gradient slice; an out-of-range offset drops the update.
+__device__ __forceinline__ void scatter_add(rsrc_t r, float *, uint32_t off, float v) {
+  __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(v, r, off, 0, 0);
+}
+__device__ __forceinline__ void scatter_add(rsrc_t, double *base, uint32_t off, double v) {
+  if (off < kNoChan) unsafeAtomicAdd(reinterpret_cast<double *>(reinterpret_cast<char *>(base) + off), v);
+}
+
+// ---------------------------------------------------------------------------------------
+// wave-private LDS hand-over between phases: LDS operations of one wavefront execute in
+// program order, so only the compiler has to be kept from moving accesses across the point.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ void wave_lds_handover() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ---------------------------------------------------------------------------------------
+// level table in LDS: H, W, Dd, first key; a level whose extent does not fit in the S keys
+// (or has a non-positive size) is disabled so that no access can leave the tensors.
+// ---------------------------------------------------------------------------------------
+struct LevelTable {
+  int H[DFA3D_MAX_LEVELS];
+  int W[DFA3D_MAX_LEVELS];
+  int Dd[DFA3D_MAX_LEVELS];
+  int start[DFA3D_MAX_LEVELS];
+};
+
+__device__ __forceinline__ void load_level_table(LevelTable &tab, const int64_t *shapes, int shape_stride,
+                                                 const int64_t *level_start, int L, int S, int D) {
+  if ((int)threadIdx.x < L) {
+    const int l = threadIdx.x;
+    const int64_t H = shapes[l * shape_stride], W = shapes[l * shape_stride + 1];
+    const int64_t Dd = shape_stride > 2 ? shapes[l * shape_stride + 2] : 1;
+    const int64_t st = level_start[l];
+    const bool ok = H > 0 && W > 0 && st >= 0 && H <= S && W <= S && st + H * W <= (int64_t)S &&
+                    Dd > 0 && (shape_stride <= 2 || Dd <= D);
+    tab.H[l] = ok ? (int)H : 0;
+    tab.W[l] = ok ? (int)W : 0;
+    tab.Dd[l] = ok ? (int)Dd : 0;
+    tab.start[l] = ok ? (int)st : 0;
+  }
+  __syncthreads();
+}
+
+// ---------------------------------------------------------------------------------------
+// geometry of one sampling point
+// ---------------------------------------------------------------------------------------
+// Pixel coordinate of a normalised location.  The reference evaluates
+// "loc * size - 0.5" with a separately rounded product (the product is typed float before the
+// double literal promotes the subtraction), so fused multiply-add contraction is switched off:
+// floor() and the skip predicates must see exactly that value.
+template <typename A> __device__ __forceinline__ A to_pixel(A loc, int size) {
+#pragma clang fp contract(off)
+  const A prod = loc * (A)size;
+  const A im = prod - (A)0.5;
+  return im;
+}
+
+// The reference floors with floorf() for every scalar type (a double is rounded to float first).
+template <typename A> __device__ __forceinline__ int floor_index(A x) { return (int)floorf((float)x); }
+
+template <typename A> struct Point2D {
+  A lh, lw, hh, hw;      // fractional parts and complements along h and w
+  int key[4];            // key index (level start + h*W + w) of slots LT,RT,RB,LB; -1 outside the map
+  bool inside;           // stage-2 predicate: -1 < h_im < H and -1 < w_im < W
+  __device__ __forceinline__ A bil(int k) const {
+    return k == 0 ? hh * hw : k == 1 ? hh * lw : k == 2 ? lh * lw : lh * hw;
+  }
+};
+
+template <typename A>
+__device__ __forceinline__ Point2D<A> locate_2d(A x, A y, int H, int W, int start) {
+  Point2D<A> g;
+  const A h_im = to_pixel(y, H), w_im = to_pixel(x, W);
+  g.inside = h_im > -1 && w_im > -1 && h_im < H && w_im < W;
+  const int h0 = floor_index(h_im), w0 = floor_index(w_im);
+  g.lh = h_im - h0;
+  g.lw = w_im - w0;
+  g.hh = 1 - g.lh;
+  g.hw = 1 - g.lw;
+  const bool h_lo = h0 >= 0 && h0 <= H - 1, h_hi = h0 + 1 >= 0 && h0 + 1 <= H - 1;
+  const bool w_lo = w0 >= 0 && w0 <= W - 1, w_hi = w0 + 1 >= 0 && w0 + 1 <= W - 1;
+  const int base = start + h0 * W + w0;
+  g.key[0] = (g.inside && h_lo && w_lo) ? base : -1;
+  g.key[1] = (g.inside && h_lo && w_hi) ? base + 1 : -1;
+  g.key[2] = (g.inside && h_hi && w_hi) ? base + W + 1 : -1;
+  g.key[3] = (g.inside && h_hi && w_lo) ? base + W : -1;
+  return g;
+}
+
+template <typename A> struct DepthTap {
+  A ld, hd;              // fractional part along depth and complement
+  int d0;                // lower bin
+  bool lo_ok, hi_ok;     // bins d0 / d0+1 inside [0, Dd-1]
+  bool inside;           // -1 < d_im < Dd
+};
+
+template <typename A> __device__ __forceinline__ DepthTap<A> locate_depth(A z, int Dd) {
+  DepthTap<A> t;
+  const A d_im = to_pixel(z, Dd);
+  t.inside = d_im > -1 && d_im < Dd;
+  t.d0 = floor_index(d_im);
+  t.ld = d_im - t.d0;
+  t.hd = 1 - t.ld;
+  t.lo_ok = t.inside && t.d0 >= 0 && t.d0 <= Dd - 1;
+  t.hi_ok = t.inside && t.d0 + 1 >= 0 && t.d0 + 1 <= Dd - 1;
+  return t;
+}
+
+// Depth scores of the four corners of one point: linear interpolation along depth of the
+// distribution stored at each corner pixel, zero outside the map / outside [0, Dd-1].
+// `dist_r` describes batch element b of dist; lo/hi return the two taps per corner.
+template <typename T, typename A>
+__device__ __forceinline__ void corner_scores(rsrc_t dist_r, const int (&key)[4], const DepthTap<A> &tap, int m, int M,
+                                              int D, A (&score)[4], A (&lo)[4], A (&hi)[4]) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint32_t row = (uint32_t)(((key[k] * M + m) * D + tap.d0) * (int)sizeof(T));
+    const bool on = key[k] >= 0;
+    lo[k] = BufElem<T>::ld(dist_r, (on && tap.lo_ok) ? row : kNoRow);
+    hi[k] = BufElem<T>::ld(dist_r, (on && tap.hi_ok) ? row + (uint32_t)sizeof(T) : kNoRow);
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) score[k] = lo[k] * tap.hd + hi[k] * tap.ld;
+}
+
+// one task of phase B: byte offset of a value row inside the batch element (kNoRow = nothing
+// to gather) and the weight the row is multiplied with
+template <typename A> struct Task;
+template <> struct __align__(8) Task<float> { uint32_t off; float w; };
+template <> struct __align__(16) Task<double> { uint32_t off; uint32_t pad; double w; };
+
+// how a wavefront maps onto units and points
+struct WaveShape {
+  int LP;          // points per unit
+  int upw;         // units handled together by one wavefront (1 when LP > 64)
+  int chunks;      // 64-point chunks per group of units
+};
+__host__ __device__ inline WaveShape wave_shape(int L, int P) {
+  WaveShape s;
+  s.LP = L * P;
+  s.upw = s.LP >= kWave ? 1 : kWave / s.LP;
+  if (s.upw > 8) s.upw = 8;
+  s.chunks = (s.upw * s.LP + kWave - 1) / kWave;
+  return s;
+}
+
+}  // namespace dfa3d

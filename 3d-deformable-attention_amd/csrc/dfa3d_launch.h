@@ -1,0 +1,79 @@
+// Host-side argument blocks and tiling choice shared by the launchers and the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace dfa3d {
+
+// How the 64 lanes of a wavefront cover value rows in phase B: LPR lanes of VEC channels per
+// row, 64/LPR rows per load instruction.  Channels beyond VEC*LPR are covered by extra passes.
+struct RowTiling { int vec, lpr; };
+
+#define DFA3D_ROW_TILINGS(X) \
+  X(1, 4) X(1, 16) X(1, 32) X(1, 64) X(2, 8) X(2, 16) X(2, 32) X(4, 8) X(4, 16) X(4, 32) X(4, 64)
+
+inline bool tiling_exists(int vec, int lpr) {
+#define DFA3D_HAS(V, R) if (vec == V && lpr == R) return true;
+  DFA3D_ROW_TILINGS(DFA3D_HAS)
+#undef DFA3D_HAS
+  return false;
+}
+
+// vec_hint > 0 forces that vector width when it fits the channel count.
+inline RowTiling pick_row_tiling(int C, int elem_size, int vec_hint) {
+  const int order_wide[3] = {4, 2, 1}, order_std[3] = {2, 4, 1};
+  const int *order = elem_size <= 2 ? order_wide : order_std;
+  for (int i = -1; i < 3; ++i) {
+    const int vec = i < 0 ? vec_hint : order[i];
+    if (vec != 1 && vec != 2 && vec != 4) continue;
+    if (C % vec) continue;
+    const int lpr = C / vec;
+    if ((lpr & (lpr - 1)) == 0 && tiling_exists(vec, lpr)) return RowTiling{vec, lpr};
+  }
+  return RowTiling{1, C <= 4 ? 4 : C <= 16 ? 16 : 64};
+}
+
+struct FwdArgs {
+  const void *value, *dist;          // dist == nullptr: stage 2 alone, scores read from score_in
+  const int64_t *shapes; int shape_stride;
+  const int64_t *level_start;
+  const void *loc; int loc_stride;
+  const void *attn, *score_in;
+  void *out, *score_out;             // score_out may be nullptr
+  int B, S, M, C, D, L, Q, P;
+  int iters;                         // groups of units each wavefront walks through
+  int vec_hint;
+};
+
+struct DepthScoreArgs {
+  const void *dist; const int64_t *shapes3, *level_start; const void *loc3;
+  void *score;
+  int B, S, M, D, L, Q, P;
+};
+
+struct BwdArgs {
+  const void *value, *dist;          // dist == nullptr: stage 2 alone
+  const int64_t *shapes; int shape_stride;
+  const int64_t *level_start;
+  const void *loc; int loc_stride;
+  const void *attn, *score_in, *grad_out, *grad_score_in;
+  void *grad_value, *grad_dist, *grad_loc; int grad_loc_stride;
+  void *grad_attn, *grad_score_out;
+  int B, S, M, C, D, L, Q, P;
+  int iters;
+  int vec_hint;
+};
+
+struct DepthScoreBwdArgs {
+  const void *dist; const int64_t *shapes3, *level_start; const void *loc3, *grad_score;
+  void *grad_dist, *grad_loc3;
+  int B, S, M, D, L, Q, P;
+};
+
+hipError_t launch_forward(const FwdArgs &a, int dtype, hipStream_t stream);
+hipError_t launch_depth_score(const DepthScoreArgs &a, int dtype, hipStream_t stream);
+hipError_t launch_backward(const BwdArgs &a, int dtype, hipStream_t stream);
+hipError_t launch_depth_score_backward(const DepthScoreBwdArgs &a, int dtype, hipStream_t stream);
+
+}  // namespace dfa3d

@@ -1,0 +1,82 @@
+"""ctypes binding of libdfa3d_hip.so (C ABI declared in include/dfa3d.h).
+
+The library is the product: there is no CPU or pure-PyTorch fallback.  If the
+shared object is missing or a tensor is not on a GPU, the call raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdfa3d_hip.so")
+
+DFA3D_F32, DFA3D_F64, DFA3D_BF16 = 0, 1, 2
+ABI_VERSION = 1
+
+_P, _I = ctypes.c_void_p, ctypes.c_int
+_DIMS7 = [_I] * 7      # B S M (C|D) L Q P
+_DIMS8 = [_I] * 8      # B S M C D L Q P
+
+# name -> argument types; every entry point returns int
+SIGNATURES = {
+    "dfa3d_ms_depth_score_sample_forward": [_P] * 5 + _DIMS7 + [_I, _P],
+    "dfa3d_ms_depth_score_sample_backward": [_P] * 7 + _DIMS7 + [_I, _P],
+    "dfa3d_wms_deform_attn_forward": [_P, _P, _I, _P, _P, _I, _P, _P, _P] + _DIMS7 + [_I, _P],
+    "dfa3d_wms_deform_attn_backward": [_P, _P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P] + _DIMS7 + [_I, _P],
+    "dfa3d_fused_forward": [_P] * 8 + _DIMS8 + [_I, _P],
+    "dfa3d_fused_backward": [_P] * 12 + _DIMS8 + [_I, _P],
+    "dfa3d_set_tunable": [ctypes.c_char_p, _I],
+    "dfa3d_abi_version": [],
+}
+
+_lib = None
+
+
+def lib():
+    """Loads the shared library once; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python 3d-deformable-attention_amd/build.py` "
+                "(hipcc, --offload-arch=gfx950). There is no fallback implementation.")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, argtypes in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = ctypes.c_int
+        handle.dfa3d_last_error.argtypes = []
+        handle.dfa3d_last_error.restype = ctypes.c_char_p
+        if handle.dfa3d_abi_version() != ABI_VERSION:
+            raise ImportError(f"{LIB_PATH}: ABI version {handle.dfa3d_abi_version()} != expected {ABI_VERSION}; rebuild")
+        _lib = handle
+    return _lib
+
+
+def check(rc, name):
+    if rc != 0:
+        msg = lib().dfa3d_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{name} failed with code {rc}: {msg}")
+
+
+def set_tunable(name, value):
+    check(lib().dfa3d_set_tunable(name.encode(), int(value)), "dfa3d_set_tunable")
+
+
+def dtype_code(t):
+    if t.dtype == torch.float32:
+        return DFA3D_F32
+    if t.dtype == torch.float64:
+        return DFA3D_F64
+    if t.dtype == torch.bfloat16:
+        return DFA3D_BF16
+    raise TypeError(f"DFA3D kernels take float32, float64 or bfloat16 storage, got {t.dtype}")
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def stream_of(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)

@@ -1,0 +1,213 @@
+#!/usr/bin/env python3
+"""Benchmark of the DFA3D operator on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload base|small|unit|dense|base_bf16]
+
+A step is one forward + backward of the one-stage autograd Function
+(MultiScale3DDeformableAttnFunction.apply -> torch.autograd.grad) over one batch of synthetic
+BEVFormer-shaped operands already resident in HBM.  Prints ONE JSON line:
+
+  metric/value   sampled points (B*Q*M*L*P) per second of forward+backward, whole job
+  ms_per_step    forward+backward through autograd (includes its allocations and zero fills)
+  kernels        per-kernel launch durations measured with events on the launch stream, with the
+                 algorithmic GB/s (each operand read once, each result written once) they amount to
+  roofline       the same for the dominant (longest) kernel, against MI355X's 8 TB/s HBM peak
+  cpu_baseline   the scalar C restatement of the operator (oracle/) on the host cores, on a
+                 bounded sample of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "3d-deformable-attention_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (scaled by
+# what the same counters read for a plain copy kernel of known size); see profiles/.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="base")
+    ap.add_argument("--kernel-reps", type=int, default=20, help="launches per kernel for the event timings")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--iters", type=int, default=0, help="library tunable 'iters' (0 = default)")
+    ap.add_argument("--vec", type=int, default=-1, help="library tunable 'vec' (-1 = default)")
+    return ap.parse_args()
+
+
+def event_time(fn, reps, prep=None):
+    """Average duration (ms) of fn() on the current stream, bracketed by events per launch."""
+    import torch
+    total = 0.0
+    best = float("inf")
+    for _ in range(reps):
+        if prep is not None:
+            prep()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        fn()
+        e.record()
+        e.synchronize()
+        ms = s.elapsed_time(e)
+        total += ms
+        best = min(best, ms)
+    return total / reps, best
+
+
+def cpu_baseline(w, budget_s):
+    """Forward+backward of the C restatement on a bounded sample (fewer queries, same everything else)."""
+    import torch
+    from dfa3D.workloads import make_inputs, scaled
+    from oracle import dfa3d_oracle as orc
+    threads = max(1, min(os.cpu_count() or 1, 64))
+    orc.set_threads(threads)
+    sample = scaled(w, Q=max(1, min(w.Q, 1000)))
+    inp = make_inputs(sample, seed=1234)
+    if inp["value"].dtype != torch.float32:
+        inp = {k: (v.float() if v.is_floating_point() else v) for k, v in inp.items()}
+    args = (inp["value"], inp["value_dpt_dist"], inp["spatial_shapes"], inp["level_start_index"],
+            inp["sampling_locations"], inp["attention_weights"])
+    reps, spent = 0, 0.0
+    while reps < 1 or (spent < budget_s and reps < 50):
+        t0 = time.perf_counter()
+        _, score = orc.dfa3d_forward(*args)
+        orc.dfa3d_backward(*args, score, inp["grad_output"])
+        spent += time.perf_counter() - t0
+        reps += 1
+    per_step = spent / reps
+    return {"value": sample.points / per_step, "unit": "points/s", "cores": threads, "kind": "port",
+            "sample": f"{w.name} workload with Q={sample.Q} of {w.Q} queries per batch element "
+                      f"({sample.points} points), forward+backward, {reps} repetition(s), {per_step * 1e3:.1f} ms each; "
+                      f"OpenMP over units (forward) and over the {sample.B} batch elements (backward)"}
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (one MI355X per box); --gpus {a.gpus} is not supported. "
+              "The operator shards over the batch (camera) dimension without any exchange.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from dfa3D import _ext, _lib
+    from dfa3D.functional import MultiScale3DDeformableAttnFunction
+    from dfa3D.workloads import WORKLOADS, make_inputs
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP kernels are the product and there is no fallback", file=sys.stderr)
+        sys.exit(3)
+    _lib.lib()
+    if a.iters > 0:
+        _lib.set_tunable("iters", a.iters)
+    if a.vec >= 0:
+        _lib.set_tunable("vec", a.vec)
+
+    bf16 = a.workload.endswith("_bf16")
+    wname = "base_peaky" if a.workload == "base_bf16" else a.workload
+    w = WORKLOADS[wname]
+    dev = torch.device("cuda:0")
+    inp = make_inputs(w, device=dev)
+    value, dist = inp["value"], inp["value_dpt_dist"]
+    go = inp["grad_output"]
+    if bf16:
+        value, dist, go = value.bfloat16(), dist.bfloat16(), go.bfloat16()
+    shapes, lsi = inp["spatial_shapes"], inp["level_start_index"]
+    loc, attn = inp["sampling_locations"], inp["attention_weights"]
+    e_v = 2 if bf16 else 4
+    fwd_bytes, bwd_bytes = w.forward_bytes(e_v, e_v), w.backward_bytes(e_v, e_v)
+    # the fused backward recomputes the depth scores instead of reading the saved ones
+    bwd_bytes_touched = bwd_bytes - 4 * e_v * w.points
+
+    leaves = [t.requires_grad_() for t in (value, dist, loc, attn)]
+
+    def step():
+        out, _ = MultiScale3DDeformableAttnFunction.apply(leaves[0], leaves[1], shapes, lsi, leaves[2], leaves[3], 64)
+        return torch.autograd.grad(out, leaves, go)
+
+    def fwd_only():
+        with torch.no_grad():
+            return MultiScale3DDeformableAttnFunction.apply(value, dist, shapes, lsi, loc, attn, 64)
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        fwd_only()
+    torch.cuda.synchronize()
+    fwd_api_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+
+    # ---- per-kernel durations: one launch between two events on the launch stream ----
+    aux = torch.float32
+    gv = torch.zeros(value.shape, dtype=aux, device=dev)
+    gd = torch.zeros(dist.shape, dtype=aux, device=dev)
+    gl = torch.empty_like(loc)
+    ga = torch.empty_like(attn)
+    vd, dd, ld, ad = value.detach(), dist.detach(), loc.detach(), attn.detach()
+    fwd_ms, fwd_best = event_time(lambda: _ext.dfa3d_fused_forward(vd, dd, shapes, lsi, ld, ad, 64), a.kernel_reps)
+
+    def zero():
+        gv.zero_()
+        gd.zero_()
+
+    bwd_ms, bwd_best = event_time(
+        lambda: _ext.dfa3d_fused_backward(vd, dd, shapes, lsi, ld, ad, go, None, gv, gd, gl, ga, 64),
+        a.kernel_reps, prep=zero)
+    fill_ms, _ = event_time(zero, a.kernel_reps)
+
+    def kernel_entry(name, ms, best, nbytes):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        return {"kernel": name, "avg_ms": round(ms, 4), "min_ms": round(best, 4),
+                "algorithmic_bytes": nbytes, "achieved_gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+                "points_per_s": w.points / (ms * 1e-3)}
+
+    kernels = {
+        "forward": kernel_entry("fwd_attention_kernel (fused depth score + attention)", fwd_ms, fwd_best, fwd_bytes),
+        "backward": kernel_entry("bwd_attention_kernel (fused)", bwd_ms, bwd_best, bwd_bytes),
+    }
+    dom = "backward" if bwd_ms >= fwd_ms else "forward"
+    k = kernels[dom]
+    roofline = {"bound": "hbm", "kernel": k["kernel"], "achieved": k["achieved_gbs"], "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": k["frac_of_hbm_peak"], "traffic": MEASURED_TRAFFIC_BYTES.get((a.workload, dom))}
+
+    result = {
+        "metric": "dfa3d_fwd_bwd_sampled_points_per_s",
+        "value": w.points / (ms_per_step * 1e-3),
+        "unit": "points/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if bf16 else "f32", "data": "synthetic",
+        "config": {"workload": f"{a.workload}: B={w.B} Q={w.Q} M={w.M} C={w.C} L={w.L} "
+                               f"levels={'/'.join(f'{h}x{x}' for h, x in w.levels)} D={w.D} P={w.P} "
+                               f"({w.points} sampled points), one-stage Function forward+backward"},
+        "fwd_ms": round(fwd_api_ms, 4), "fwd_kernel_ms": round(fwd_ms, 4), "bwd_kernel_ms": round(bwd_ms, 4),
+        "grad_zero_fill_ms": round(fill_ms, 4),
+        "fwd_frac_of_hbm_peak": kernels["forward"]["frac_of_hbm_peak"],
+        "bwd_bytes_actually_touched": bwd_bytes_touched,
+        "kernels": kernels,
+        "roofline": roofline,
+    }
+    if a.cpu_seconds > 0:
+        result["cpu_baseline"] = cpu_baseline(w, a.cpu_seconds)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,122 @@
+/*
+ * libdfa3d_hip - DFA3D (3D deformable attention) operator for AMD MI355X (gfx950).
+ *
+ * C ABI of the shared library.  Every pointer except `stream` is a DEVICE pointer
+ * into memory the caller owns; the library allocates nothing, keeps no state
+ * besides a thread-local error string, launches on `stream` (a hipStream_t, NULL
+ * = the default stream) and returns without synchronising.  Return value: 0 on
+ * success, a negative DFA3D_E* code for a rejected argument, a positive
+ * hipError_t for a failed launch; dfa3d_last_error() describes the last failure
+ * of the calling thread.
+ *
+ * Tensor layouts (all contiguous, row-major), with
+ *   B batch, S = sum_l H_l*W_l keys, M heads, C channels per head, D depth bins,
+ *   L levels, Q queries, P points per level:
+ *     value        (B,S,M,C)            dist        (B,S,M,D)
+ *     shapes       (L,shape_stride) int64, row = (H, W[, Dd]); shape_stride is 2 or 3
+ *     level_start  (L) int64, first key of each level
+ *     loc          (B,Q,M,L,P,loc_stride), (x, y[, z]) normalised to [0,1]; loc_stride 2 or 3
+ *     attn         (B,Q,M,L,P)          score       (B,Q,M,L,P,4)  slots LT,RT,RB,LB
+ *     out          (B,Q,M*C)
+ *
+ * dtype selects the element types:
+ *     DFA3D_F32   every floating tensor float
+ *     DFA3D_F64   every floating tensor double
+ *     DFA3D_BF16  value, dist, out, score are bfloat16; loc, attn and EVERY gradient
+ *                 buffer are float (accumulation is float throughout)
+ *
+ * The four *_forward / *_backward pairs replace the reference's four native entry
+ * points one for one; the two dfa3d_fused_* calls run both stages in one kernel.
+ */
+#ifndef DFA3D_H
+#define DFA3D_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DFA3D_F32 0
+#define DFA3D_F64 1
+#define DFA3D_BF16 2
+
+#define DFA3D_MAX_LEVELS 16
+
+#define DFA3D_EINVAL (-1)   /* null pointer, non-positive dimension, bad stride or dtype */
+#define DFA3D_ERANGE (-2)   /* a dimension exceeds what the kernels index (see dfa3d_last_error) */
+
+/* Stage 1 forward: multi-scale depth-score sampling.  Writes every element of `score`.
+ * Replaces ms_depth_score_sample_forward
+ * (DFA3D/dfa3D/ops/csrc/pybind.cpp:55-59 ->
+ *  DFA3D/dfa3D/ops/csrc/cuda/ms_depth_score_sample_cuda.cu:49-111). */
+int dfa3d_ms_depth_score_sample_forward(
+    const void *dist, const int64_t *shapes3, const int64_t *level_start, const void *loc3,
+    void *score,
+    int B, int S, int M, int D, int L, int Q, int P, int dtype, void *stream);
+
+/* Stage 1 backward.  `grad_dist` is ACCUMULATED into (caller zero-fills); every element of
+ * `grad_loc3` is overwritten, its x and y components with 0.
+ * Replaces ms_depth_score_sample_backward
+ * (pybind.cpp:60-66 -> ms_depth_score_sample_cuda.cu:137-202). */
+int dfa3d_ms_depth_score_sample_backward(
+    const void *dist, const int64_t *shapes3, const int64_t *level_start, const void *loc3,
+    const void *grad_score,
+    void *grad_dist, void *grad_loc3,
+    int B, int S, int M, int D, int L, int Q, int P, int dtype, void *stream);
+
+/* Stage 2 forward: depth-weighted multi-scale deformable attention.  Writes every element of
+ * `out`.  Replaces wms_deform_attn_forward
+ * (pybind.cpp:43-47 -> DFA3D/dfa3D/ops/csrc/cuda/wms_deform_attn_cuda.cu:213-288). */
+int dfa3d_wms_deform_attn_forward(
+    const void *value, const int64_t *shapes, int shape_stride, const int64_t *level_start,
+    const void *loc, int loc_stride, const void *attn, const void *score,
+    void *out,
+    int B, int S, int M, int C, int L, int Q, int P, int dtype, void *stream);
+
+/* Stage 2 backward.  `grad_value` is ACCUMULATED into (caller zero-fills); `grad_loc`
+ * (B,Q,M,L,P,grad_loc_stride) gets its first two components overwritten, `grad_attn` and
+ * `grad_score` are overwritten.  Replaces wms_deform_attn_backward
+ * (pybind.cpp:48-54 -> wms_deform_attn_cuda.cu:291-370). */
+int dfa3d_wms_deform_attn_backward(
+    const void *value, const int64_t *shapes, int shape_stride, const int64_t *level_start,
+    const void *loc, int loc_stride, const void *attn, const void *score, const void *grad_out,
+    void *grad_value, void *grad_loc, int grad_loc_stride, void *grad_attn, void *grad_score,
+    int B, int S, int M, int C, int L, int Q, int P, int dtype, void *stream);
+
+/* Both stages in one kernel: what the reference's one-stage autograd Function does with two
+ * native calls and two slice copies
+ * (BEVFormer_DFA3D/projects/mmdet3d_plugin/bevformer/modules/multi_scale_3ddeformable_attn_function.py:279-303).
+ * Writes every element of `out` and, when `score` is not NULL, of `score`. */
+int dfa3d_fused_forward(
+    const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
+    const void *loc3, const void *attn,
+    void *out, void *score,
+    int B, int S, int M, int C, int D, int L, int Q, int P, int dtype, void *stream);
+
+/* Backward of dfa3d_fused_forward (…_function.py:306-352: two native calls, six zero fills and
+ * a host synchronisation in the reference).  The depth scores are recomputed from `dist`, not
+ * read back.  `grad_score_in` (may be NULL) is an incoming gradient with respect to the `score`
+ * output and is chained into grad_dist and the z gradient.  `grad_value` and `grad_dist` are
+ * ACCUMULATED into (caller zero-fills); `grad_loc3` and `grad_attn` are overwritten. */
+int dfa3d_fused_backward(
+    const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
+    const void *loc3, const void *attn, const void *grad_out, const void *grad_score_in,
+    void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn,
+    int B, int S, int M, int C, int D, int L, int Q, int P, int dtype, void *stream);
+
+/* Message for the last non-zero return on the calling thread ("" if none). */
+const char *dfa3d_last_error(void);
+
+/* Process-wide launch tunables; results do not depend on them.
+ *   "iters"  groups of units each wavefront walks through (default 1)
+ *   "vec"    channels per lane in the row gathers: 0 = automatic, 1, 2 or 4 */
+int dfa3d_set_tunable(const char *name, int value);
+
+/* Library ABI version (bumped when a signature changes). */
+int dfa3d_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DFA3D_H */

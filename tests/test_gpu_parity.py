@@ -1,0 +1,276 @@
+"""GPU parity: the HIP kernels, called through the autograd Functions (and so through the C ABI),
+against the CPU checker on identical seeded inputs.
+
+Tolerances (stated by the task): fp32 forward rtol = atol = 1e-5; fp32 backward rtol = atol = 1e-4
+(floating-point atomics make the summation order of grad_value / grad_dist nondeterministic);
+fp64 1e-10 / 1e-11 forward / backward; bf16 storage: see test_bf16_storage.
+"""
+import pytest
+import torch
+
+from forms import tiny_case
+
+pytestmark = pytest.mark.gpu
+
+F32_FWD = dict(rtol=1e-5, atol=1e-5)
+F32_BWD = dict(rtol=1e-4, atol=1e-4)
+
+
+def _dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return torch.device("cuda:0")
+
+
+def _functions():
+    from dfa3D.ops.multi_scale_3D_deform_attn import (MultiScale3DDeformableAttnFunction,
+                                                      MultiScaleDepthScoreSampleFunction,
+                                                      WeightedMultiScaleDeformableAttnFunction)
+    return MultiScale3DDeformableAttnFunction, MultiScaleDepthScoreSampleFunction, \
+        WeightedMultiScaleDeformableAttnFunction
+
+
+def _gpu_one_stage(inp, dev, grad_score=None):
+    F1, _, _ = _functions()
+    value = inp["value"].to(dev).requires_grad_()
+    dist = inp["value_dpt_dist"].to(dev).requires_grad_()
+    loc = inp["sampling_locations"].to(dev).requires_grad_()
+    attn = inp["attention_weights"].to(dev).requires_grad_()
+    out, score = F1.apply(value, dist, inp["spatial_shapes"].to(dev), inp["level_start_index"].to(dev), loc, attn, 64)
+    outs, gouts = [out], [inp["grad_output"].to(dev)]
+    if grad_score is not None:
+        outs.append(score)
+        gouts.append(grad_score.to(dev))
+    gv, gd, gl, ga = torch.autograd.grad(outs, [value, dist, loc, attn], gouts)
+    torch.cuda.synchronize()
+    return out.detach().cpu(), score.detach().cpu(), gv.cpu(), gd.cpu(), gl.cpu(), ga.cpu()
+
+
+def _oracle_one_stage(oracle, inp):
+    out, score = oracle.dfa3d_forward(inp["value"], inp["value_dpt_dist"], inp["spatial_shapes"],
+                                      inp["level_start_index"], inp["sampling_locations"], inp["attention_weights"])
+    gv, gd, gl, ga = oracle.dfa3d_backward(inp["value"], inp["value_dpt_dist"], inp["spatial_shapes"],
+                                           inp["level_start_index"], inp["sampling_locations"],
+                                           inp["attention_weights"], score, inp["grad_output"])
+    return out, score, gv, gd, gl, ga
+
+
+def _as_inputs(t):
+    return {"value": t["value"], "value_dpt_dist": t["dist"], "spatial_shapes": t["shapes3"],
+            "level_start_index": t["lsi"], "sampling_locations": t["loc"], "attention_weights": t["attn"],
+            "grad_output": t["grad_out"]}
+
+
+def _compare(got, want, fwd_tol, bwd_tol):
+    names = ["output", "depth_score", "grad_value", "grad_dist", "grad_loc", "grad_attn"]
+    for i, (g, w, n) in enumerate(zip(got, want, names)):
+        tol = fwd_tol if i < 2 else bwd_tol
+        torch.testing.assert_close(g, w, msg=lambda m, n=n: f"{n}: {m}", **tol)
+
+
+TINY = [
+    dict(seed=0),                                                    # C=3 (generic row tiling), L*P=6
+    dict(seed=1, C=32, M=8, Q=5, P=8, levels=((6, 9), (4, 5), (3, 3), (2, 2))),   # L*P=32, C=32 fast path
+    dict(seed=2, C=64, M=4, Q=3, P=4, levels=((5, 5),)),             # single level, C=64
+    dict(seed=3, C=16, M=3, Q=2, P=30, levels=((4, 6), (2, 3), (3, 2))),          # L*P=90 > 64: chunked units
+    dict(seed=4, C=5, M=1, Q=9, P=1, levels=((3, 4),)),              # L*P=1
+    dict(seed=5, C=128, M=2, Q=2, P=2, levels=((4, 4), (2, 2)), D=1),             # D=1
+    dict(seed=6, C=100, M=2, Q=3, P=3, levels=((4, 4), (2, 3))),     # C not a power of two, > 64: two passes
+    dict(seed=7, C=256, M=1, Q=2, P=2, levels=((3, 3),)),
+]
+
+
+@pytest.mark.parametrize("case", TINY, ids=lambda c: "-".join(f"{k}{v}" for k, v in c.items() if k != "levels"))
+def test_fp64_one_stage_matches_checker(oracle, case):
+    dev = _dev()
+    inp = _as_inputs(tiny_case(**case))
+    got = _gpu_one_stage(inp, dev)
+    want = _oracle_one_stage(oracle, inp)
+    _compare(got, want, dict(rtol=1e-10, atol=1e-11), dict(rtol=1e-10, atol=1e-11))
+
+
+@pytest.mark.parametrize("case", TINY[:4], ids=lambda c: f"seed{c['seed']}")
+def test_fp32_one_stage_matches_checker_tiny(oracle, case):
+    dev = _dev()
+    t = tiny_case(**case)
+    inp = {k: (v.float() if v.is_floating_point() else v) for k, v in _as_inputs(t).items()}
+    _compare(_gpu_one_stage(inp, dev), _oracle_one_stage(oracle, inp), F32_FWD, F32_BWD)
+
+
+def test_fp64_two_stage_matches_checker_and_chains(oracle):
+    dev = _dev()
+    _, F3, F2 = _functions()
+    t = tiny_case(11, C=32, M=4, Q=6, P=4, levels=((5, 7), (3, 4)))
+    inp = _as_inputs(t)
+    dist = inp["value_dpt_dist"].to(dev).requires_grad_()
+    value = inp["value"].to(dev).requires_grad_()
+    loc3 = inp["sampling_locations"].to(dev).requires_grad_()
+    attn = inp["attention_weights"].to(dev).requires_grad_()
+    shapes3, lsi = inp["spatial_shapes"].to(dev), inp["level_start_index"].to(dev)
+    score = F3.apply(dist, shapes3, lsi, loc3, 64)
+    out = F2.apply(value, shapes3[:, :2].contiguous(), lsi, loc3[..., :2].contiguous(), attn, score, 64)
+    gv, gd, gl, ga = torch.autograd.grad(out, [value, dist, loc3, attn], inp["grad_output"].to(dev))
+    want = _oracle_one_stage(oracle, inp)
+    got = (out.detach().cpu(), score.detach().cpu(), gv.cpu(), gd.cpu(), gl.cpu(), ga.cpu())
+    _compare(got, want, dict(rtol=1e-10, atol=1e-11), dict(rtol=1e-10, atol=1e-11))
+
+
+def test_fp64_stage2_alone_arbitrary_scores(oracle):
+    dev = _dev()
+    _, _, F2 = _functions()
+    t = tiny_case(12, C=32, M=2, Q=4, P=4, levels=((5, 7), (3, 4)))
+    g = torch.Generator().manual_seed(3)
+    score = torch.randn(*t["loc"].shape[:-1], 4, generator=g, dtype=torch.float64)
+    shapes2 = t["shapes3"][:, :2].contiguous()
+    loc2 = t["loc"][..., :2].contiguous()
+    leaves = [x.to(dev).requires_grad_() for x in (t["value"], loc2, t["attn"], score)]
+    out = F2.apply(leaves[0], shapes2.to(dev), t["lsi"].to(dev), leaves[1], leaves[2], leaves[3], 64)
+    gv, gl, ga, gs = torch.autograd.grad(out, leaves, t["grad_out"].to(dev))
+    o_out = oracle.wms_forward(t["value"], shapes2, t["lsi"], loc2, t["attn"], score)
+    o_gv, o_gl, o_ga, o_gs = oracle.wms_backward(t["value"], shapes2, t["lsi"], loc2, t["attn"], score, t["grad_out"])
+    tol = dict(rtol=1e-10, atol=1e-11)
+    for a, b in ((out, o_out), (gv, o_gv), (gl, o_gl), (ga, o_ga), (gs, o_gs)):
+        torch.testing.assert_close(a.detach().cpu(), b, **tol)
+
+
+def test_fp64_stage1_alone_backward(oracle):
+    dev = _dev()
+    _, F3, _ = _functions()
+    t = tiny_case(13, M=3, Q=6, P=5, D=7, levels=((5, 7), (3, 4)))
+    g = torch.Generator().manual_seed(4)
+    gsc = torch.randn(*t["loc"].shape[:-1], 4, generator=g, dtype=torch.float64)
+    dist = t["dist"].to(dev).requires_grad_()
+    loc = t["loc"].to(dev).requires_grad_()
+    score = F3.apply(dist, t["shapes3"].to(dev), t["lsi"].to(dev), loc, 64)
+    gd, gl = torch.autograd.grad(score, [dist, loc], gsc.to(dev))
+    o_gd, o_gl = oracle.depth_score_backward(t["dist"], t["shapes3"], t["lsi"], t["loc"], gsc)
+    tol = dict(rtol=1e-10, atol=1e-11)
+    torch.testing.assert_close(score.detach().cpu(), oracle.depth_score_forward(t["dist"], t["shapes3"], t["lsi"], t["loc"]), **tol)
+    torch.testing.assert_close(gd.cpu(), o_gd, **tol)
+    torch.testing.assert_close(gl.cpu(), o_gl, **tol)
+    assert gl[..., :2].abs().max().item() == 0
+
+
+def test_gradient_through_depth_score_output(oracle):
+    """A gradient arriving at the depth_score output is chained (the reference refuses it)."""
+    dev = _dev()
+    t = tiny_case(14, C=32, M=2, Q=4, P=4, levels=((5, 7), (3, 4)))
+    inp = _as_inputs(t)
+    g = torch.Generator().manual_seed(8)
+    gsc = torch.randn(*t["loc"].shape[:-1], 4, generator=g, dtype=torch.float64)
+    got = _gpu_one_stage(inp, dev, grad_score=gsc)
+    want = list(_oracle_one_stage(oracle, inp))
+    extra_gd, extra_gl = oracle.depth_score_backward(t["dist"], t["shapes3"], t["lsi"], t["loc"], gsc)
+    want[3] = want[3] + extra_gd
+    want[4] = want[4] + extra_gl
+    _compare(got, want, dict(rtol=1e-10, atol=1e-11), dict(rtol=1e-10, atol=1e-11))
+
+
+@pytest.mark.parametrize("name", ["unit", "small"])
+def test_fp32_workloads_match_checker(oracle, name):
+    from dfa3D.workloads import WORKLOADS, make_inputs
+    dev = _dev()
+    inp = make_inputs(WORKLOADS[name])
+    _compare(_gpu_one_stage(inp, dev), _oracle_one_stage(oracle, inp), F32_FWD, F32_BWD)
+
+
+def test_fp32_base_shape_matches_checker(oracle):
+    """BEVFormer-base shape at full size (15.36 M sampling points)."""
+    from dfa3D.workloads import WORKLOADS, make_inputs
+    dev = _dev()
+    inp = make_inputs(WORKLOADS["base"])
+    got = _gpu_one_stage(inp, dev)
+    want = _oracle_one_stage(oracle, inp)
+    _compare(got, want, F32_FWD, F32_BWD)
+
+
+def _inner(a, b):
+    return (a.double() * b.double()).sum().item()
+
+
+def test_fp32_dense_shape_properties():
+    """Dense BEV stress shape (61.44 M points), too big for the scalar checker in seconds:
+    size-independent identities.  The operator is linear in value, in the depth distributions and
+    in the attention weights, so <x, dL/dx> = <output, grad_output> for each of them (Euler), and
+    the two-stage chain must reproduce the one-stage result."""
+    from dfa3D.workloads import WORKLOADS, make_inputs
+    dev = _dev()
+    F1, F3, F2 = _functions()
+    inp = make_inputs(WORKLOADS["dense"], device=dev)
+    value = inp["value"].requires_grad_()
+    dist = inp["value_dpt_dist"].requires_grad_()
+    loc = inp["sampling_locations"]
+    attn = inp["attention_weights"].requires_grad_()
+    shapes3, lsi = inp["spatial_shapes"], inp["level_start_index"]
+    out, score = F1.apply(value, dist, shapes3, lsi, loc, attn, 64)
+    go = inp["grad_output"]
+    gv, gd, ga = torch.autograd.grad(out, [value, dist, attn], go)
+    ref = _inner(out, go)
+    scale = (out.double().abs() * go.double().abs()).sum().item()
+    for name, x, gx in (("value", value, gv), ("dist", dist, gd), ("attn", attn, ga)):
+        assert abs(_inner(x, gx) - ref) <= 1e-5 * scale, name
+    with torch.no_grad():
+        score2 = F3.apply(dist.detach(), shapes3, lsi, loc, 64)
+        assert torch.equal(score2, score)
+        out2 = F2.apply(value.detach(), shapes3[:, :2].contiguous(), lsi, loc[..., :2].contiguous(),
+                        attn.detach(), score2, 64)
+        torch.testing.assert_close(out2, out.detach(), **F32_FWD)
+        # linearity in value at full size
+        out3, _ = F1.apply(value.detach() * 2 + 1, dist.detach(), shapes3, lsi, loc, attn.detach(), 64)
+        ones, _ = F1.apply(torch.ones_like(value), dist.detach(), shapes3, lsi, loc, attn.detach(), 64)
+        torch.testing.assert_close(out3, 2 * out.detach() + ones, rtol=1e-4, atol=1e-5)
+
+
+def test_bf16_storage(oracle):
+    """bfloat16 value / distributions (peaky, GT-depth-like), float32 locations and weights, float32
+    accumulation.  Checked against the fp32 checker run on the bf16-ROUNDED inputs: the only extra
+    error is the bf16 rounding of the stored outputs (output, depth_score: 2^-8 relative) and of the
+    returned value / dist gradients; grad_loc and grad_attn stay float32."""
+    from dfa3D.workloads import WORKLOADS, make_inputs, scaled
+    dev = _dev()
+    F1, _, _ = _functions()
+    w = scaled(WORKLOADS["base_peaky"], B=2, Q=1500)
+    inp = make_inputs(w, seed=4)
+    v16, d16 = inp["value"].bfloat16(), inp["value_dpt_dist"].bfloat16()
+    go16 = inp["grad_output"].bfloat16()
+    value, dist = v16.to(dev).requires_grad_(), d16.to(dev).requires_grad_()
+    loc, attn = inp["sampling_locations"].to(dev).requires_grad_(), inp["attention_weights"].to(dev).requires_grad_()
+    out, score = F1.apply(value, dist, inp["spatial_shapes"].to(dev), inp["level_start_index"].to(dev), loc, attn, 64)
+    assert out.dtype == torch.bfloat16 and score.dtype == torch.bfloat16
+    gv, gd, gl, ga = torch.autograd.grad(out, [value, dist, loc, attn], go16.to(dev))
+    assert gv.dtype == torch.bfloat16 and gd.dtype == torch.bfloat16 and gl.dtype == torch.float32
+    ref = dict(inp, value=v16.float(), value_dpt_dist=d16.float(), grad_output=go16.float())
+    o_out, o_score, o_gv, o_gd, o_gl, o_ga = _oracle_one_stage(oracle, ref)
+    bf = dict(rtol=8e-3, atol=8e-3)
+    torch.testing.assert_close(out.float().cpu(), o_out, **bf)
+    torch.testing.assert_close(score.float().cpu(), o_score, **bf)
+    torch.testing.assert_close(gv.float().cpu(), o_gv, **bf)
+    torch.testing.assert_close(gd.float().cpu(), o_gd, rtol=8e-3, atol=8e-3 * max(1.0, o_gd.abs().max().item()))
+    torch.testing.assert_close(gl.cpu(), o_gl, **F32_BWD)
+    torch.testing.assert_close(ga.cpu(), o_ga, **F32_BWD)
+
+
+def test_nan_in_unsampled_pixel_does_not_leak(oracle):
+    """Corners outside the map are never read and never multiplied in."""
+    dev = _dev()
+    t = tiny_case(20, C=32, M=1, Q=3, P=2, levels=((4, 4),), lo=0.3, hi=0.7)
+    inp = _as_inputs(t)
+    inp["value"][:, 0] = float("nan")          # pixel (0, 0): no location in [0.3, 0.7]^2 touches it
+    inp["sampling_locations"][0, 0, 0, 0, 0, :2] = torch.tensor([1.1, 0.5], dtype=torch.float64)   # RT/RB outside
+    got = _gpu_one_stage(inp, dev)
+    want = _oracle_one_stage(oracle, inp)
+    assert torch.isfinite(got[0]).all()
+    torch.testing.assert_close(got[0], want[0], rtol=1e-10, atol=1e-11)
+
+
+def test_inconsistent_level_table_is_contained():
+    """A level that does not fit in the key dimension is treated as empty instead of reading out of
+    bounds (the reference would read past the tensor)."""
+    dev = _dev()
+    F1, _, _ = _functions()
+    t = tiny_case(21, C=32, M=2, Q=4, P=2, levels=((4, 4), (2, 2)))
+    bad = t["shapes3"].clone()
+    bad[1, 0] = 50                       # 50 x 2 keys do not fit
+    out, score = F1.apply(t["value"].to(dev), t["dist"].to(dev), bad.to(dev), t["lsi"].to(dev),
+                          t["loc"].to(dev), t["attn"].to(dev), 64)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all() and score[:, :, :, 1].abs().max().item() == 0
