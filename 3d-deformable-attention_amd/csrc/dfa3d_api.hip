@@ -35,6 +35,7 @@ int env_int(const char *name, int dflt) {
 }
 std::atomic<int> g_iters{env_int("DFA3D_ITERS", 1)};
 std::atomic<int> g_vec{env_int("DFA3D_VEC", 0)};
+std::atomic<int> g_diag{0};
 int tune_iters() { const int v = g_iters.load(std::memory_order_relaxed); return v < 1 ? 1 : v; }
 int tune_vec() { return g_vec.load(std::memory_order_relaxed); }
 
@@ -60,9 +61,29 @@ int check_dims(const char *fn, int B, int S, int M, int width, int L, int Q, int
 #define REQUIRE_PTR(fn, p) \
   if ((p) == nullptr) return fail(DFA3D_EINVAL, "%s: %s is NULL", fn, #p)
 
+// Plain streaming copy, 16 bytes per lane: the yardstick the profiler's HBM counters are scaled by.
+__global__ __launch_bounds__(256) void stream_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
+                                                          size_t n16) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
 }  // namespace
 
 extern "C" {
+
+int dfa3d_stream_copy(void *dst, const void *src, size_t bytes, void *stream) {
+  const char *fn = "dfa3d_stream_copy";
+  REQUIRE_PTR(fn, dst); REQUIRE_PTR(fn, src);
+  if (bytes == 0 || bytes % 16 != 0 || ((uintptr_t)dst | (uintptr_t)src) % 16 != 0)
+    return fail(DFA3D_EINVAL, "%s: size and both pointers must be non-zero multiples of 16 bytes", fn);
+  const size_t n16 = bytes / 16;
+  size_t blocks = (n16 + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const uint4 *)src, (uint4 *)dst, n16);
+  return hip_result(hipGetLastError(), fn);
+}
 
 const char *dfa3d_last_error(void) { return g_err; }
 int dfa3d_abi_version(void) { return 1; }
@@ -78,6 +99,10 @@ int dfa3d_set_tunable(const char *name, int value) {
     if (value != 0 && value != 1 && value != 2 && value != 4)
       return fail(DFA3D_EINVAL, "dfa3d_set_tunable: vec must be 0 (automatic), 1, 2 or 4");
     g_vec.store(value, std::memory_order_relaxed);
+    return 0;
+  }
+  if (!strcmp(name, "diag")) {
+    g_diag.store(value, std::memory_order_relaxed);
     return 0;
   }
   return fail(DFA3D_EINVAL, "dfa3d_set_tunable: unknown tunable '%s'", name);
@@ -142,7 +167,7 @@ int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int
   a.grad_score_in = nullptr; a.grad_value = grad_value; a.grad_dist = nullptr; a.grad_loc = grad_loc;
   a.grad_loc_stride = grad_loc_stride; a.grad_attn = grad_attn; a.grad_score_out = grad_score;
   a.B = B; a.S = S; a.M = M; a.C = C; a.D = 1; a.L = L; a.Q = Q; a.P = P;
-  a.iters = tune_iters(); a.vec_hint = tune_vec();
+  a.iters = tune_iters(); a.vec_hint = tune_vec(); a.diag = g_diag.load(std::memory_order_relaxed);
   return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
 }
 
@@ -178,7 +203,7 @@ int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *sha
   a.grad_score_in = grad_score_in; a.grad_value = grad_value; a.grad_dist = grad_dist; a.grad_loc = grad_loc3;
   a.grad_loc_stride = 3; a.grad_attn = grad_attn; a.grad_score_out = nullptr;
   a.B = B; a.S = S; a.M = M; a.C = C; a.D = D; a.L = L; a.Q = Q; a.P = P;
-  a.iters = tune_iters(); a.vec_hint = tune_vec();
+  a.iters = tune_iters(); a.vec_hint = tune_vec(); a.diag = g_diag.load(std::memory_order_relaxed);
   return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
 }
 

@@ -124,7 +124,7 @@ __global__ __launch_bounds__(kBlock) void bwd_attention_kernel(
     const A *__restrict__ attn, const T *__restrict__ score_in, const T *__restrict__ grad_out,
     const T *__restrict__ grad_score_in, A *__restrict__ grad_value, A *__restrict__ grad_dist,
     A *__restrict__ grad_loc, int gl_stride, A *__restrict__ grad_attn, A *__restrict__ grad_score_out,
-    int B, int S, int M, int C, int D, int L, int Q, int P, int iters, int q_blocks) {
+    int B, int S, int M, int C, int D, int L, int Q, int P, int iters, int q_blocks, int diag) {
   __shared__ LevelTable tab;
   __shared__ Task<A> s_tasks[kWavesPerBlock][kWave * 4];
   __shared__ A s_dots[kWavesPerBlock][kWave * 4];
@@ -144,10 +144,10 @@ __global__ __launch_bounds__(kBlock) void bwd_attention_kernel(
   A *gvalue_b = grad_value + (size_t)b * S * M * C;
   A *gdist_b = FUSED ? grad_dist + (size_t)b * S * M * D : nullptr;
   const rsrc_t value_r = make_rsrc(value + (size_t)b * S * M * C, (size_t)S * M * C * sizeof(T));
-  const rsrc_t gvalue_r = make_rsrc(gvalue_b, (size_t)S * M * C * sizeof(A));
+  const rsrc_t gvalue_r = make_rsrc(gvalue_b, (diag & 1) ? 0 : (size_t)S * M * C * sizeof(A));
   const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * M * D : nullptr,
                                   FUSED ? (size_t)S * M * D * sizeof(T) : 0);
-  const rsrc_t gdist_r = make_rsrc(gdist_b, FUSED ? (size_t)S * M * D * sizeof(A) : 0);
+  const rsrc_t gdist_r = make_rsrc(gdist_b, (FUSED && !(diag & 2)) ? (size_t)S * M * D * sizeof(A) : 0);
   const int q_per_iter = kWavesPerBlock * ws.upw;
 
   for (int it = 0; it < iters; ++it) {
@@ -334,14 +334,14 @@ static hipError_t launch_bwd_cfg(const BwdArgs &a, hipStream_t stream) {
                        (const A *)a.loc, a.loc_stride, (const A *)a.attn, (const T *)nullptr,
                        (const T *)a.grad_out, (const T *)a.grad_score_in, (A *)a.grad_value, (A *)a.grad_dist,
                        (A *)a.grad_loc, a.grad_loc_stride, (A *)a.grad_attn, (A *)nullptr, a.B, a.S, a.M, a.C, a.D,
-                       a.L, a.Q, a.P, iters, q_blocks);
+                       a.L, a.Q, a.P, iters, q_blocks, a.diag);
   } else {
     hipLaunchKernelGGL((bwd_attention_kernel<T, A, VEC, LPR, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,
                        (const T *)a.value, (const T *)nullptr, a.shapes, a.shape_stride, a.level_start,
                        (const A *)a.loc, a.loc_stride, (const A *)a.attn, (const T *)a.score_in,
                        (const T *)a.grad_out, (const T *)nullptr, (A *)a.grad_value, (A *)nullptr, (A *)a.grad_loc,
                        a.grad_loc_stride, (A *)a.grad_attn, (A *)a.grad_score_out, a.B, a.S, a.M, a.C, a.D, a.L, a.Q,
-                       a.P, iters, q_blocks);
+                       a.P, iters, q_blocks, a.diag);
   }
   return hipGetLastError();
 }

@@ -63,6 +63,7 @@ struct BwdArgs {
   int B, S, M, C, D, L, Q, P;
   int iters;
   int vec_hint;
+  int diag;                          // measurement aid: bit 0 drops the grad_value updates, bit 1 the grad_dist updates
 };
 
 struct DepthScoreBwdArgs {

@@ -27,6 +27,7 @@ SIGNATURES = {
     "dfa3d_fused_forward": [_P] * 8 + _DIMS8 + [_I, _P],
     "dfa3d_fused_backward": [_P] * 12 + _DIMS8 + [_I, _P],
     "dfa3d_set_tunable": [ctypes.c_char_p, _I],
+    "dfa3d_stream_copy": [_P, _P, ctypes.c_size_t, _P],
     "dfa3d_abi_version": [],
 }
 

@@ -40,6 +40,8 @@ def parse():
     ap.add_argument("--workload", default="base")
     ap.add_argument("--kernel-reps", type=int, default=20, help="launches per kernel for the event timings")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--calibration-copy-mib", type=int, default=0,
+                    help="also run one plain streaming copy of this many MiB (yardstick for profiler HBM counters)")
     ap.add_argument("--iters", type=int, default=0, help="library tunable 'iters' (0 = default)")
     ap.add_argument("--vec", type=int, default=-1, help="library tunable 'vec' (-1 = default)")
     return ap.parse_args()
@@ -126,6 +128,16 @@ def main():
     fwd_bytes, bwd_bytes = w.forward_bytes(e_v, e_v), w.backward_bytes(e_v, e_v)
     # the fused backward recomputes the depth scores instead of reading the saved ones
     bwd_bytes_touched = bwd_bytes - 4 * e_v * w.points
+
+    if a.calibration_copy_mib > 0:
+        n = a.calibration_copy_mib << 20
+        src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(2):
+            _lib.check(_lib.lib().dfa3d_stream_copy(_lib.ptr(dst), _lib.ptr(src), n, _lib.stream_of(src)),
+                       "dfa3d_stream_copy")
+        torch.cuda.synchronize()
+        del src, dst
 
     leaves = [t.requires_grad_() for t in (value, dist, loc, attn)]
 

@@ -3,7 +3,7 @@
  *
  * C ABI of the shared library.  Every pointer except `stream` is a DEVICE pointer
  * into memory the caller owns; the library allocates nothing, keeps no state
- * besides a thread-local error string, launches on `stream` (a hipStream_t, NULL
+ * besides a thread-local error string and the launch tunables, launches on `stream` (a hipStream_t, NULL
  * = the default stream) and returns without synchronising.  Return value: 0 on
  * success, a negative DFA3D_E* code for a rejected argument, a positive
  * hipError_t for a failed launch; dfa3d_last_error() describes the last failure
@@ -31,6 +31,7 @@
 #ifndef DFA3D_H
 #define DFA3D_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -110,8 +111,14 @@ const char *dfa3d_last_error(void);
 
 /* Process-wide launch tunables; results do not depend on them.
  *   "iters"  groups of units each wavefront walks through (default 1)
- *   "vec"    channels per lane in the row gathers: 0 = automatic, 1, 2 or 4 */
+ *   "vec"    channels per lane in the row gathers: 0 = automatic, 1, 2 or 4
+ *   "diag"   measurement aid for the backward kernels: bit 0 drops the grad_value updates,
+ *            bit 1 the grad_dist updates (results are then incomplete); default 0 */
 int dfa3d_set_tunable(const char *name, int value);
+
+/* Measurement aid: copies `bytes` (a multiple of 16, 16-byte aligned pointers) from src to dst with
+ * a plain streaming kernel.  It is the copy of known size that profiler HBM counters are scaled by. */
+int dfa3d_stream_copy(void *dst, const void *src, size_t bytes, void *stream);
 
 /* Library ABI version (bumped when a signature changes). */
 int dfa3d_abi_version(void);
