@@ -36,6 +36,10 @@ int env_int(const char *name, int dflt) {
 std::atomic<int> g_iters{env_int("DFA3D_ITERS", 1)};
 std::atomic<int> g_vec{env_int("DFA3D_VEC", 0)};
 std::atomic<int> g_diag{0};
+std::atomic<int> g_tile{0};
+std::atomic<int> g_block{0};
+std::atomic<int> g_chunk{0};
+std::atomic<int> g_binned{1};
 int tune_iters() { const int v = g_iters.load(std::memory_order_relaxed); return v < 1 ? 1 : v; }
 int tune_vec() { return g_vec.load(std::memory_order_relaxed); }
 
@@ -86,7 +90,7 @@ int dfa3d_stream_copy(void *dst, const void *src, size_t bytes, void *stream) {
 }
 
 const char *dfa3d_last_error(void) { return g_err; }
-int dfa3d_abi_version(void) { return 1; }
+int dfa3d_abi_version(void) { return 2; }
 
 int dfa3d_set_tunable(const char *name, int value) {
   if (name == nullptr) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: name is NULL");
@@ -99,6 +103,29 @@ int dfa3d_set_tunable(const char *name, int value) {
     if (value != 0 && value != 1 && value != 2 && value != 4)
       return fail(DFA3D_EINVAL, "dfa3d_set_tunable: vec must be 0 (automatic), 1, 2 or 4");
     g_vec.store(value, std::memory_order_relaxed);
+    return 0;
+  }
+  if (!strcmp(name, "tile")) {
+    const int ty = value / 100, tx = value % 100;
+    if (value != 0 && (ty < 1 || tx < 1 || ty > 64 || tx > 64))
+      return fail(DFA3D_EINVAL, "dfa3d_set_tunable: tile must be 0 or ty*100+tx with 1 <= ty, tx <= 64");
+    g_tile.store(value, std::memory_order_relaxed);
+    return 0;
+  }
+  if (!strcmp(name, "block")) {
+    if (value != 0 && (value < 64 || value > 1024 || value % 64 != 0))
+      return fail(DFA3D_EINVAL, "dfa3d_set_tunable: block must be 0 or a multiple of 64 in [64, 1024]");
+    g_block.store(value, std::memory_order_relaxed);
+    return 0;
+  }
+  if (!strcmp(name, "chunk")) {
+    if (value != 0 && (value < 64 || value > (1 << 20)))
+      return fail(DFA3D_EINVAL, "dfa3d_set_tunable: chunk must be 0 or in [64, 2^20]");
+    g_chunk.store(value, std::memory_order_relaxed);
+    return 0;
+  }
+  if (!strcmp(name, "binned")) {
+    g_binned.store(value != 0, std::memory_order_relaxed);
     return 0;
   }
   if (!strcmp(name, "diag")) {
@@ -187,16 +214,11 @@ int dfa3d_fused_forward(const void *value, const void *dist, const int64_t *shap
   return hip_result(dfa3d::launch_forward(a, dtype, (hipStream_t)stream), fn);
 }
 
-int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
-                         const void *loc3, const void *attn, const void *grad_out, const void *grad_score_in,
-                         void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn, int B, int S, int M,
-                         int C, int D, int L, int Q, int P, int dtype, void *stream) {
-  const char *fn = "dfa3d_fused_backward";
-  if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
-  if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
-  REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
-  REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
-  REQUIRE_PTR(fn, grad_dist); REQUIRE_PTR(fn, grad_loc3); REQUIRE_PTR(fn, grad_attn);
+static dfa3d::BwdArgs fused_bwd_args(const void *value, const void *dist, const int64_t *shapes3,
+                                     const int64_t *level_start, const void *loc3, const void *attn,
+                                     const void *grad_out, const void *grad_score_in, void *grad_value,
+                                     void *grad_dist, void *grad_loc3, void *grad_attn, int B, int S, int M, int C,
+                                     int D, int L, int Q, int P) {
   dfa3d::BwdArgs a{};
   a.value = value; a.dist = dist; a.shapes = shapes3; a.shape_stride = 3; a.level_start = level_start;
   a.loc = loc3; a.loc_stride = 3; a.attn = attn; a.score_in = nullptr; a.grad_out = grad_out;
@@ -204,6 +226,37 @@ int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *sha
   a.grad_loc_stride = 3; a.grad_attn = grad_attn; a.grad_score_out = nullptr;
   a.B = B; a.S = S; a.M = M; a.C = C; a.D = D; a.L = L; a.Q = Q; a.P = P;
   a.iters = tune_iters(); a.vec_hint = tune_vec(); a.diag = g_diag.load(std::memory_order_relaxed);
+  a.tile_hint = g_tile.load(std::memory_order_relaxed); a.block_hint = g_block.load(std::memory_order_relaxed);
+  a.chunk_hint = g_chunk.load(std::memory_order_relaxed);
+  return a;
+}
+
+size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, int L, int Q, int P, int dtype) {
+  if (check_dims("dfa3d_fused_backward_workspace_bytes", B, S, M, C, L, Q, P, dtype)) return 0;
+  if (check_dims("dfa3d_fused_backward_workspace_bytes", B, S, M, D, L, Q, P, dtype)) return 0;
+  if (!g_binned.load(std::memory_order_relaxed)) return 0;
+  const dfa3d::BwdArgs a = fused_bwd_args(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                                          nullptr, nullptr, nullptr, nullptr, B, S, M, C, D, L, Q, P);
+  return dfa3d::binned_backward_workspace_bytes(a, dtype);
+}
+
+int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
+                         const void *loc3, const void *attn, const void *grad_out, const void *grad_score_in,
+                         void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn,
+                         void *workspace, size_t workspace_bytes, int B, int S, int M,
+                         int C, int D, int L, int Q, int P, int dtype, void *stream) {
+  const char *fn = "dfa3d_fused_backward";
+  if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
+  if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
+  REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
+  REQUIRE_PTR(fn, grad_dist); REQUIRE_PTR(fn, grad_loc3); REQUIRE_PTR(fn, grad_attn);
+  const dfa3d::BwdArgs a = fused_bwd_args(value, dist, shapes3, level_start, loc3, attn, grad_out, grad_score_in,
+                                          grad_value, grad_dist, grad_loc3, grad_attn, B, S, M, C, D, L, Q, P);
+  if (workspace != nullptr && g_binned.load(std::memory_order_relaxed)) {
+    const hipError_t e = dfa3d::launch_backward_binned(a, dtype, workspace, workspace_bytes, (hipStream_t)stream);
+    if (e != hipErrorNotSupported) return hip_result(e, fn);
+  }
   return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
 }
 

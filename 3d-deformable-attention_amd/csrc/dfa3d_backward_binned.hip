@@ -1,0 +1,700 @@
+// Binned backward of the fused DFA3D operator for gfx950: no floating-point atomics on device
+// memory in the hot loop.
+//
+// Why: device-memory atomics retire at roughly 10^10 cache-line requests per second on this part,
+// and the straightforward backward (bwd_attention_kernel) needs 4 row updates of grad_value and 8
+// scalar updates of grad_dist per sampling point.  LDS atomics are two orders of magnitude faster.
+// So the points are first binned by the image tile they fall in, and one workgroup per tile
+// accumulates that tile of grad_value and grad_dist in LDS and writes it out once.
+//
+//   plan_and_clear_kernel  validates the level table, lays out the tiles (bins), clears counters
+//   bin_count_kernel       points per bin (LDS histogram per block, one atomic per touched bin)
+//   bin_scan_kernel        exclusive prefix over bins
+//   bin_fill_kernel        writes each point's index into its bin's segment; zero gradients for
+//                          points the operator skips
+//   tile_backward_kernel   persistent workgroups pull (bin, chunk of its points) work items from a
+//                          queue; per item: LDS tiles
+//                          of (TY+1) x (TX+1) pixels (one-pixel halo to the right/bottom, so all four
+//                          corners of a point of this bin land in the tile), the same three phases
+//                          as the direct kernel with LDS atomics, then one flush of the tile
+//
+// A point belongs to the tile that holds its clamped base pixel (clamp(h0,0,H-1), clamp(w0,0,W-1)).
+// Semantics are those of bwd_attention_kernel (see dfa3d_backward.hip for the formulas and the
+// reference lines they restate).
+#include "dfa3d_device.h"
+#include "dfa3d_launch.h"
+
+namespace dfa3d {
+
+constexpr int kQueues = 1;          // work-queue counters in the workspace
+constexpr int kBinQueries = 64;     // queries of one (batch, head) handled by a count/fill block
+constexpr int kHistCap = 8192;      // bins of one (batch, head) that fit the LDS histogram
+
+struct BinPlan {
+  int H[DFA3D_MAX_LEVELS], W[DFA3D_MAX_LEVELS], Dd[DFA3D_MAX_LEVELS], start[DFA3D_MAX_LEVELS];
+  int tiles_x[DFA3D_MAX_LEVELS], level_base[DFA3D_MAX_LEVELS];
+  int bins_per_bm;     // tiles over all levels of one (batch, head)
+  int total_bins;      // B * M * bins_per_bm
+  int ty, tx;          // tile edge in pixels
+  int chunk;           // points of a bin handled by one work item
+  int total_chunks;    // work items (written by the scan)
+};
+
+struct BinWorkspace {      // device pointers into the caller's workspace
+  BinPlan *plan;
+  int *queues;             // kQueues counters
+  int *counts;             // points per bin
+  int *cursor;             // begin of each bin's segment after the scan, end after the fill
+  int *chunk_end;          // inclusive prefix of work items per bin
+  uint32_t *entries;       // point indices grouped by bin
+  float4 *recs;            // (x, y, z, attention weight) of the same points, same order
+};
+
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void plan_and_clear_kernel(
+    BinWorkspace ws, const int64_t *__restrict__ shapes3, const int64_t *__restrict__ level_start, int L, int S, int D,
+    int B, int M, int ty, int tx, int chunk, int max_bins_per_bm) {
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    BinPlan p;
+    int base = 0;
+    for (int l = 0; l < DFA3D_MAX_LEVELS; ++l) {
+      int64_t H = 0, W = 0, Dd = 0, st = 0;
+      bool ok = false;
+      if (l < L) {
+        H = shapes3[l * 3]; W = shapes3[l * 3 + 1]; Dd = shapes3[l * 3 + 2]; st = level_start[l];
+        ok = H > 0 && W > 0 && st >= 0 && H <= S && W <= S && st + H * W <= (int64_t)S && Dd > 0 && Dd <= D;
+      }
+      p.H[l] = ok ? (int)H : 0; p.W[l] = ok ? (int)W : 0; p.Dd[l] = ok ? (int)Dd : 0; p.start[l] = ok ? (int)st : 0;
+      const int nx = ok ? ((int)W + tx - 1) / tx : 0, ny = ok ? ((int)H + ty - 1) / ty : 0;
+      p.tiles_x[l] = nx;
+      p.level_base[l] = base;
+      base += nx * ny;
+    }
+    // the host sized the counters from an upper bound of the tile count; never exceed it
+    if (base > max_bins_per_bm) base = 0;
+    p.bins_per_bm = base;
+    p.total_bins = base * B * M;
+    p.ty = ty; p.tx = tx;
+    p.chunk = chunk; p.total_chunks = 0;
+    *ws.plan = p;
+  }
+  const size_t n = (size_t)max_bins_per_bm * B * M;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    ws.counts[i] = 0;
+    ws.cursor[i] = 0;
+  }
+  if (blockIdx.x == 0 && threadIdx.x < 64) ws.queues[threadIdx.x] = 0;    // the counters and their padding
+}
+
+// bin (within one (batch, head)) of a point that the operator does not skip
+__device__ __forceinline__ int bin_of(const BinPlan &p, int l, const Point2D<float> &g) {
+  const int cy = min(max(g.h0, 0), p.H[l] - 1), cx = min(max(g.w0, 0), p.W[l] - 1);
+  return p.level_base[l] + (cy / p.ty) * p.tiles_x[l] + cx / p.tx;
+}
+
+// MODE 0: count.  MODE 1: fill (needs the scanned cursor).
+template <int MODE>
+__global__ __launch_bounds__(256) void bin_points_kernel(
+    BinWorkspace ws, const float *__restrict__ loc3, const float *__restrict__ attn, float *__restrict__ grad_loc3,
+    float *__restrict__ grad_attn, int B, int M, int L, int Q, int P, int q_blocks, int hist_cap) {
+  extern __shared__ int s_hist[];          // [0, nb): counts, then for MODE 1 [nb, 2 nb): segment bases
+  const BinPlan &p = *ws.plan;
+  const int nb = p.bins_per_bm;
+  if (nb == 0) return;
+  const bool use_lds = nb <= hist_cap;
+  const int bm = blockIdx.x / q_blocks, qb = blockIdx.x - bm * q_blocks;
+  const int b = bm / M, m = bm - b * M;
+  const int LP = L * P;
+  const int q0 = qb * kBinQueries, nq = min(kBinQueries, Q - q0);
+  const int npts = nq * LP;
+  int *gcount = ws.counts + (size_t)bm * nb;
+  int *gcursor = ws.cursor + (size_t)bm * nb;
+
+  if (use_lds) {
+    for (int i = threadIdx.x; i < nb * (MODE == 1 ? 2 : 1); i += blockDim.x) s_hist[i] = 0;
+    __syncthreads();
+  }
+  // pass 1: histogram of this block's points
+  for (int i = threadIdx.x; i < npts; i += blockDim.x) {
+    const int qi = i / LP, lp = i - qi * LP, l = lp / P;
+    const size_t gp = ((size_t)(b * (size_t)Q + q0 + qi) * M + m) * LP + lp;
+    const Point2D<float> g = locate_2d<float>(loc3[gp * 3], loc3[gp * 3 + 1], p.H[l], p.W[l], p.start[l]);
+    if (g.inside && p.tiles_x[l] > 0) {
+      const int bin = bin_of(p, l, g);
+      if (use_lds) atomicAdd(&s_hist[bin], 1);
+      else if (MODE == 0) atomicAdd(&gcount[bin], 1);
+    } else if (MODE == 1) {
+      // skipped by the operator: all its gradients are zero, and no tile will visit it
+      grad_loc3[gp * 3] = 0; grad_loc3[gp * 3 + 1] = 0; grad_loc3[gp * 3 + 2] = 0;
+      grad_attn[gp] = 0;
+    }
+  }
+  if (use_lds) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < nb; i += blockDim.x) {
+      const int c = s_hist[i];
+      if (c > 0) {
+        if (MODE == 0) atomicAdd(&gcount[i], c);
+        else s_hist[nb + i] = atomicAdd(&gcursor[i], c);     // reserve a run of the bin's segment
+      }
+      if (MODE == 1) s_hist[i] = 0;                          // reused as the running rank
+    }
+    __syncthreads();
+  }
+  if (MODE == 1) {
+    // pass 2: place the points
+    for (int i = threadIdx.x; i < npts; i += blockDim.x) {
+      const int qi = i / LP, lp = i - qi * LP, l = lp / P;
+      const size_t gp = ((size_t)(b * (size_t)Q + q0 + qi) * M + m) * LP + lp;
+      const Point2D<float> g = locate_2d<float>(loc3[gp * 3], loc3[gp * 3 + 1], p.H[l], p.W[l], p.start[l]);
+      if (g.inside && p.tiles_x[l] > 0) {
+        const int bin = bin_of(p, l, g);
+        const int slot = use_lds ? s_hist[nb + bin] + atomicAdd(&s_hist[bin], 1) : atomicAdd(&gcursor[bin], 1);
+        ws.entries[slot] = (uint32_t)gp;
+        ws.recs[slot] = make_float4(loc3[gp * 3], loc3[gp * 3 + 1], loc3[gp * 3 + 2], attn[gp]);
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws) {
+  __shared__ int s_pts[1024], s_chk[1024];
+  const int n = ws.plan->total_bins, ch = ws.plan->chunk;
+  const int per = (n + 1023) / 1024;
+  const int lo = min(n, (int)threadIdx.x * per), hi = min(n, lo + per);
+  int pts = 0, chk = 0;
+  for (int i = lo; i < hi; ++i) {
+    const int c = ws.counts[i];
+    pts += c;
+    chk += (c + ch - 1) / ch;
+  }
+  s_pts[threadIdx.x] = pts;
+  s_chk[threadIdx.x] = chk;
+  __syncthreads();
+  // inclusive scans of the 1024 partial sums (Hillis-Steele, a barrier pair per step)
+  for (int off = 1; off < 1024; off <<= 1) {
+    const int ap = threadIdx.x >= (unsigned)off ? s_pts[threadIdx.x - off] : 0;
+    const int ac = threadIdx.x >= (unsigned)off ? s_chk[threadIdx.x - off] : 0;
+    __syncthreads();
+    s_pts[threadIdx.x] += ap;
+    s_chk[threadIdx.x] += ac;
+    __syncthreads();
+  }
+  int run_p = s_pts[threadIdx.x] - pts, run_c = s_chk[threadIdx.x] - chk;
+  for (int i = lo; i < hi; ++i) {
+    const int c = ws.counts[i];
+    ws.cursor[i] = run_p;
+    run_p += c;
+    run_c += (c + ch - 1) / ch;
+    ws.chunk_end[i] = run_c;
+  }
+  if (threadIdx.x == 1023) ws.plan->total_chunks = s_chk[1023];
+}
+
+// ---------------------------------------------------------------------------------------
+// Tile workgroups.
+//
+// A work item is one bin (image tile of one batch element, head and level) and up to `chunk` of
+// its points.  The points are taken kTilePoints at a time (one per thread):
+//   phase A  thread = point: geometry, depth taps, corner weights; every corner becomes a task
+//            (tile row, weight, point slot); the point's grad_out row is staged in LDS
+//   sort     tasks are grouped by tile row (counting sort in LDS, integer counters)
+//   rows     a group of LPR lanes owns a tile row: it loads the value row once, then for each of the
+//            row's tasks takes the staged grad_out row, leaves the dot product for phase C and
+//            accumulates weight * grad_out in registers; the row sum is added to the LDS tile with a
+//            plain read-modify-write (nobody else touches that row during the pass)
+//   phase C  thread = point: per-point gradients from the four dots; grad_dist taps go to the LDS
+//            tile with atomics (8 scalars per point)
+// After the item's last pass the tile is flushed to memory once (atomic adds: chunks of one bin
+// and the halos of neighbouring bins overlap).
+// ---------------------------------------------------------------------------------------
+constexpr int kTilePoints = 256;     // points per pass = threads per tile workgroup
+
+// Optional phase timing of the tile kernel (development builds only, -DDFA3D_TILE_TIMING): thread 0
+// of every workgroup accumulates shader-clock ticks per phase and adds them to 64-bit counters that
+// live in the padding behind the queue counter.
+#ifdef DFA3D_TILE_TIMING
+#define TT_DECL unsigned long long tt_acc[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long tt_last = clock64();
+#define TT_MARK(i) do { if (threadIdx.x == 0) { const unsigned long long tt_now = clock64(); tt_acc[i] += tt_now - tt_last; tt_last = tt_now; } } while (0)
+#define TT_FLUSH() do { if (threadIdx.x == 0) { unsigned long long *tt_g = reinterpret_cast<unsigned long long *>(ws.queues + 16); for (int i = 0; i < 10; ++i) atomicAdd(tt_g + i, tt_acc[i]); } } while (0)
+#else
+#define TT_DECL
+#define TT_MARK(i) do { } while (0)
+#define TT_FLUSH() do { } while (0)
+#endif
+
+struct TileLds {      // offsets (in 4-byte words) into the dynamic LDS block
+  int gv, gd, gstage, tasks, dots, cnt, offs, goff, total;
+};
+__host__ __device__ inline TileLds tile_lds_layout(int ty, int tx, int C, int D) {
+  TileLds o;
+  const int R = (ty + 1) * (tx + 1);
+  o.gv = 0;
+  o.gd = o.gv + R * C;
+  o.gstage = (o.gd + R * D + 3) & ~3;              // 16-byte aligned rows
+  o.tasks = (o.gstage + kTilePoints * C + 1) & ~1; // 8-byte records
+  o.dots = o.tasks + kTilePoints * 4 * 2;
+  o.cnt = o.dots + kTilePoints * 4;
+  o.offs = o.cnt + R;
+  o.goff = o.offs + R + 1;
+  o.total = o.goff + kTilePoints;
+  return o;
+}
+
+struct RowTask { float w; uint32_t who; };   // who = point slot | corner << 16
+
+__device__ __forceinline__ float dpp_xadd(float x, int pick) {
+  const int xi = __float_as_int(x);
+  int r;
+  switch (pick) {
+    case 0: r = __builtin_amdgcn_mov_dpp(xi, 0xB1, 0xF, 0xF, true); break;    // quad_perm [1,0,3,2]
+    case 1: r = __builtin_amdgcn_mov_dpp(xi, 0x4E, 0xF, 0xF, true); break;    // quad_perm [2,3,0,1]
+    case 2: r = __builtin_amdgcn_mov_dpp(xi, 0x141, 0xF, 0xF, true); break;   // row_half_mirror
+    default: r = __builtin_amdgcn_mov_dpp(xi, 0x140, 0xF, 0xF, true); break;  // row_mirror
+  }
+  return x + __int_as_float(r);
+}
+template <int LPR> __device__ __forceinline__ float row_sum_f(float x) {
+  if (LPR >= 2) x = dpp_xadd(x, 0);
+  if (LPR >= 4) x = dpp_xadd(x, 1);
+  if (LPR >= 8) x = dpp_xadd(x, 2);
+  if (LPR >= 16) x = dpp_xadd(x, 3);
+  if (LPR >= 32) x += __shfl_xor(x, 16, kWave);
+  if (LPR >= 64) x += __shfl_xor(x, 32, kWave);
+  return x;
+}
+
+// VEC consecutive floats of an LDS row
+template <int VEC> __device__ __forceinline__ void lds_ld(const float *p, float (&v)[VEC]) {
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) v[i] = p[i];
+}
+
+template <typename T, int VEC, int LPR>
+__global__ __launch_bounds__(512) void tile_backward_kernel(
+    BinWorkspace ws, const T *__restrict__ value, const T *__restrict__ dist, const float *__restrict__ loc3,
+    const float *__restrict__ attn, const T *__restrict__ grad_out, const T *__restrict__ grad_score_in,
+    float *__restrict__ grad_value, float *__restrict__ grad_dist, float *__restrict__ grad_loc3,
+    float *__restrict__ grad_attn, int B, int S, int M, int C, int D, int L, int Q, int P, int diag) {
+  constexpr int RPI = kWave / LPR;                  // row groups per wavefront
+  extern __shared__ float smem[];
+  __shared__ int s_bin, s_item;
+
+  const BinPlan &p = *ws.plan;
+  const int nb = p.bins_per_bm;
+  if (nb == 0) return;
+  const int TY = p.ty, TX = p.tx, TW = TX + 1, R = (TY + 1) * TW;
+  const TileLds lay = tile_lds_layout(TY, TX, C, D);
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int n_thr = blockDim.x, n_waves = n_thr / kWave;
+  const int kGroups = n_waves * RPI;                   // row groups in the workgroup
+  const int stage_per_wave = kTilePoints / n_waves;    // grad_out rows each wavefront stages
+  float *gv = smem + lay.gv, *gd = smem + lay.gd, *gstage = smem + lay.gstage, *dots = smem + lay.dots;
+  RowTask *tasks = reinterpret_cast<RowTask *>(smem + lay.tasks);
+  int *cnt = reinterpret_cast<int *>(smem + lay.cnt), *offs = reinterpret_cast<int *>(smem + lay.offs);
+  uint32_t *goff = reinterpret_cast<uint32_t *>(smem + lay.goff);
+  const int group = wave * RPI + lane / LPR, cl = lane % LPR;
+  const int passes = (C + VEC * LPR - 1) / (VEC * LPR);
+  const int LP = L * P;
+
+  for (int i = tid; i < R * (C + D); i += n_thr) smem[i] = 0;   // gv and gd are adjacent
+  TT_DECL
+
+  const int total_bins = p.total_bins, total_chunks = p.total_chunks, CH = p.chunk;
+  for (;;) {
+    // ---- next work item: (bin, chunk of its points), in bin order
+    __syncthreads();
+    if (tid == 0) {
+      const int w = atomicAdd(&ws.queues[0], 1);
+      int bin = -1;
+      if (w < total_chunks) {
+        int lo = 0, hi = total_bins - 1;               // first bin whose inclusive chunk prefix exceeds w
+        while (lo < hi) {
+          const int mid = (lo + hi) >> 1;
+          if (ws.chunk_end[mid] > w) hi = mid; else lo = mid + 1;
+        }
+        bin = lo;
+      }
+      s_bin = bin;
+      s_item = w;
+    }
+    __syncthreads();
+    const int bin = s_bin;
+    if (bin < 0) break;                                   // queue drained: every wave leaves
+    TT_MARK(0);
+    const int n_bin = ws.counts[bin];
+    const int chunks_here = (n_bin + CH - 1) / CH;
+    const int chunk_id = s_item - (ws.chunk_end[bin] - chunks_here);
+    const int first = chunk_id * CH;
+    const int n_item = min(CH, n_bin - first);
+    const int seg = ws.cursor[bin] - n_bin + first;       // the fill advanced the cursor to the segment's end
+    const int bm = bin / nb, local = bin - bm * nb;
+    const int b = bm / M, m = bm - b * M;
+    int l = 0;
+    while (l + 1 < L && local >= p.level_base[l + 1]) ++l;
+    const int tile = local - p.level_base[l];
+    const int H = p.H[l], W = p.W[l], Dd = p.Dd[l], start = p.start[l];
+    const int y0 = (tile / p.tiles_x[l]) * TY, x0 = (tile % p.tiles_x[l]) * TX;
+
+    const rsrc_t value_r = make_rsrc(value + (size_t)b * S * M * C, (size_t)S * M * C * sizeof(T));
+    const rsrc_t dist_r = make_rsrc(dist + (size_t)b * S * M * D, (size_t)S * M * D * sizeof(T));
+    const rsrc_t go_r = make_rsrc(grad_out + (size_t)b * Q * M * C, (size_t)Q * M * C * sizeof(T));
+
+    for (int base = 0; base < n_item; base += kTilePoints) {      // uniform over the workgroup
+      const int cnt_pts = min(kTilePoints, n_item - base);
+      // ---------------- phase A: one thread per point ----------------
+      for (int i = tid; i < R; i += n_thr) cnt[i] = 0;
+      const bool live = tid < cnt_pts;
+      size_t gp = 0;
+      Point2D<float> g;
+      DepthTap<float> tap;
+      float a = 0, sc[4], lo[4], hi[4], wk[4];
+      int tr[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) { tr[k] = -1; wk[k] = 0; sc[k] = 0; lo[k] = 0; hi[k] = 0; g.key[k] = -1; }
+      g.inside = false; g.lh = g.lw = g.hh = g.hw = 0; g.h0 = g.w0 = 0;
+      tap.inside = tap.lo_ok = tap.hi_ok = false; tap.d0 = 0; tap.ld = tap.hd = 0;
+      uint32_t my_goff = kNoRow;
+      if (live) {
+        gp = ws.entries[seg + base + tid];
+        const float4 rec = ws.recs[seg + base + tid];
+        const size_t unit = gp / LP;
+        a = rec.w;
+        g = locate_2d<float>(rec.x, rec.y, H, W, start);
+        tap = locate_depth<float>(rec.z, Dd);
+        corner_scores<T, float>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
+        my_goff = (uint32_t)((unit - (size_t)b * Q * M) * C * sizeof(T));
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (g.key[k] >= 0) {
+            const int ry = g.h0 + (k >= 2 ? 1 : 0) - y0, rx = g.w0 + ((k == 1 || k == 2) ? 1 : 0) - x0;
+            if (ry >= 0 && ry <= TY && rx >= 0 && rx <= TX) {
+              tr[k] = ry * TW + rx;
+              wk[k] = g.bil(k) * sc[k] * a;
+            }
+          }
+        }
+      }
+      if (tid < kTilePoints) goff[tid] = my_goff;
+      __syncthreads();                                   // counters cleared, goff visible
+      TT_MARK(1);
+      int rank[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) rank[k] = tr[k] >= 0 ? atomicAdd(&cnt[tr[k]], 1) : 0;
+      // stage the grad_out rows of this wavefront's 64 points (lanes over channels)
+      for (int pass = 0; pass < passes; ++pass) {
+        const int chan = (pass * LPR + cl) * VEC;
+        const uint32_t chan_off = chan < C ? (uint32_t)(chan * sizeof(T)) : kNoChan;
+#pragma unroll 4
+        for (int j = 0; j < stage_per_wave; j += RPI) {
+          const int slot = wave * stage_per_wave + j + lane / LPR;
+          float gg[VEC];
+          RowVec<T, float, VEC>::ld(go_r, goff[slot] + chan_off, gg);
+          if (chan < C) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) gstage[slot * C + chan + i] = gg[i];
+          }
+        }
+      }
+      __syncthreads();                                   // counts complete
+      TT_MARK(2);
+      if (wave == 0) {                                   // exclusive prefix of the row counters
+        int run = 0;
+        for (int r0 = 0; r0 < R; r0 += kWave) {
+          const int r = r0 + lane;
+          const int c = r < R ? cnt[r] : 0;
+          int inc = c;
+#pragma unroll
+          for (int off = 1; off < kWave; off <<= 1) {
+            const int up = __shfl_up(inc, off, kWave);
+            if (lane >= off) inc += up;
+          }
+          if (r < R) offs[r] = run + inc - c;
+          run += __shfl(inc, kWave - 1, kWave);
+        }
+        if (lane == 0) offs[R] = run;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (tid >= kTilePoints) {
+        } else if (tr[k] >= 0) {
+          RowTask t;
+          t.w = wk[k];
+          t.who = (uint32_t)tid | ((uint32_t)k << 16);
+          tasks[offs[tr[k]] + rank[k]] = t;
+        } else {
+          dots[tid * 4 + k] = 0;                         // no row will write this dot
+        }
+      }
+      __syncthreads();                                   // tasks grouped by row, grad_out rows staged
+      TT_MARK(3);
+
+      // ---------------- rows: one group of LPR lanes per tile row ----------------
+      for (int pass = 0; pass < passes; ++pass) {
+        const int chan = (pass * LPR + cl) * VEC;
+        const bool chan_ok = chan < C;
+        const uint32_t chan_off = chan_ok ? (uint32_t)(chan * sizeof(T)) : kNoChan;
+        float v_next[VEC];
+        {
+          const int r = group;
+          const int y = y0 + r / TW, x = x0 + r % TW;
+          const bool ld_ok = r < R && offs[min(r, R - 1) + 1] > offs[min(r, R - 1)] && y < H && x < W && !(diag & 8);
+          RowVec<T, float, VEC>::ld(value_r, (ld_ok ? (uint32_t)(((start + y * W + x) * M + m) * C * (int)sizeof(T)) : kNoRow) + chan_off, v_next);
+        }
+        for (int r0 = 0; r0 < R; r0 += kGroups) {        // uniform over the workgroup
+          const int r = r0 + group;
+          const bool row_ok = r < R;
+          const int beg = row_ok ? offs[r] : 0;
+          const int n_r = row_ok ? offs[r + 1] - beg : 0;
+          int n_max = n_r;                               // longest list among this wavefront's groups
+#pragma unroll
+          for (int off = LPR; off < kWave; off <<= 1) n_max = max(n_max, __shfl_xor(n_max, off, kWave));
+          const int y = y0 + r / TW, x = x0 + r % TW;
+          const bool pix_ok = row_ok && n_r > 0 && y < H && x < W;
+          float v[VEC], acc[VEC];
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) { v[i] = v_next[i]; acc[i] = 0; }
+          {                                              // value row of this group's next round
+            const int rn = r + kGroups;
+            const int yn = y0 + rn / TW, xn = x0 + rn % TW;
+            const bool ld_ok = rn < R && offs[min(rn, R - 1) + 1] > offs[min(rn, R - 1)] && yn < H && xn < W && !(diag & 8);
+            RowVec<T, float, VEC>::ld(value_r, (ld_ok ? (uint32_t)(((start + yn * W + xn) * M + m) * C * (int)sizeof(T)) : kNoRow) + chan_off, v_next);
+          }
+          if (n_max == 0) continue;                      // wave-uniform
+          constexpr int UT = 4;
+          for (int t0 = 0; t0 < n_max; t0 += UT) {
+            RowTask tk[UT];
+            float gg[UT][VEC], part[UT];
+#pragma unroll
+            for (int j = 0; j < UT; ++j) tk[j] = tasks[min(beg + min(t0 + j, max(n_r - 1, 0)), kTilePoints * 4 - 1)];
+#pragma unroll
+            for (int j = 0; j < UT; ++j) lds_ld<VEC>(gstage + (tk[j].who & (kTilePoints - 1)) * C + (chan_ok ? chan : 0), gg[j]);
+#pragma unroll
+            for (int j = 0; j < UT; ++j) {
+              part[j] = 0;
+#pragma unroll
+              for (int i = 0; i < VEC; ++i) part[j] += v[i] * gg[j][i];
+            }
+#pragma unroll
+            for (int j = 0; j < UT; ++j) part[j] = row_sum_f<LPR>(part[j]);
+#pragma unroll
+            for (int j = 0; j < UT; ++j) {
+              if (t0 + j < n_r) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[i] += tk[j].w * gg[j][i];
+                if (cl == 0) {
+                  const int di = (tk[j].who & 0xFFFF) * 4 + (tk[j].who >> 16);
+                  dots[di] = pass == 0 ? part[j] : dots[di] + part[j];
+                }
+              }
+            }
+          }
+          if (pix_ok && chan_ok && !(diag & 1)) {
+            float *dst = gv + r * C + chan;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) dst[i] += acc[i];
+          }
+        }
+      }
+      __syncthreads();                                   // dots complete
+      TT_MARK(4);
+
+      // ---------------- phase C: per-point gradients, grad_dist taps into the LDS tile ----------------
+      if (live) {
+        float gs[4], s[4], ga = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const float dk = dots[tid * 4 + k];
+          const bool on = g.key[k] >= 0;
+          const float bk = g.bil(k);
+          gs[k] = on ? bk * a * dk : 0.f;
+          s[k] = on ? sc[k] * dk : 0.f;
+          ga += bk * s[k];
+        }
+        const float gx = (float)W * a * (g.hh * (s[1] - s[0]) + g.lh * (s[2] - s[3]));
+        const float gy = (float)H * a * (g.hw * (s[3] - s[0]) + g.lw * (s[2] - s[1]));
+        if (grad_score_in != nullptr) {
+          const T *gi = grad_score_in + gp * 4;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) gs[k] += Elem<T>::ld(gi + k);
+        }
+        float gz = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (tr[k] >= 0 && tap.inside && gs[k] != 0 && !(diag & 2)) {
+            float *dst = gd + tr[k] * D + tap.d0;
+            if (tap.lo_ok) atomicAdd(dst, tap.hd * gs[k]);
+            if (tap.hi_ok) atomicAdd(dst + 1, tap.ld * gs[k]);
+          }
+          gz += (g.key[k] >= 0 && tap.inside) ? gs[k] * (hi[k] - lo[k]) : 0.f;
+        }
+        float *gl = grad_loc3 + gp * 3;
+        gl[0] = gx; gl[1] = gy; gl[2] = gz * (float)Dd;
+        grad_attn[gp] = ga;
+      }
+      __syncthreads();                                   // before the next pass reuses the scratch arrays
+      TT_MARK(5);
+    }
+
+    // ---------------- flush the tile (and leave it zeroed for the next item) ----------------
+    float *gvalue_b = grad_value + (size_t)b * S * M * C;
+    float *gdist_b = grad_dist + (size_t)b * S * M * D;
+    const rsrc_t gvalue_r = make_rsrc(gvalue_b, (size_t)S * M * C * sizeof(float));
+    const rsrc_t gdist_r = make_rsrc(gdist_b, (size_t)S * M * D * sizeof(float));
+    for (int i = tid; i < R * C; i += n_thr) {
+      const float val = gv[i];
+      if (val != 0) {
+        gv[i] = 0;
+        const int r = i / C, c = i - r * C;
+        const int y = y0 + r / TW, x = x0 + r % TW;
+        if (y < H && x < W && !(diag & 4)) scatter_add(gvalue_r, gvalue_b, (uint32_t)((((start + y * W + x) * M + m) * C + c) * 4), val);
+      }
+    }
+    for (int i = tid; i < R * D; i += n_thr) {
+      const float val = gd[i];
+      if (val != 0) {
+        gd[i] = 0;
+        const int r = i / D, d = i - r * D;
+        const int y = y0 + r / TW, x = x0 + r % TW;
+        if (y < H && x < W && !(diag & 4)) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * M + m) * D + d) * 4), val);
+      }
+    }
+    TT_MARK(6);
+  }
+  TT_MARK(7);
+  TT_FLUSH();
+}
+
+// ---------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------
+static int max_bins_per_bm(int S, int L, int ty, int tx) {
+  // tiles of a level <= (H/ty + 1) (W/tx + 1) <= HW/(ty tx) + H/ty + W/tx + 1 and H + W <= HW + 1
+  const int e = ty < tx ? ty : tx;
+  const long long v = (long long)S / (ty * tx) + ((long long)S + L) / e + 2LL * L + 1;
+  return (int)v;
+}
+
+struct BinLayout { size_t plan, queues, counts, cursor, chunk_end, entries, recs, total; };
+static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
+  BinLayout o;
+  const size_t nbins = (size_t)max_bins_per_bm(a.S, a.L, ty, tx) * a.B * a.M;
+  const size_t npts = (size_t)a.B * a.Q * a.M * a.L * a.P;
+  auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
+  o.plan = 0;
+  o.queues = up(o.plan + sizeof(BinPlan));
+  o.counts = up(o.queues + kQueues * sizeof(int));
+  o.cursor = up(o.counts + nbins * sizeof(int));
+  o.chunk_end = up(o.cursor + nbins * sizeof(int));
+  o.entries = up(o.chunk_end + nbins * sizeof(int));
+  o.recs = up(o.entries + npts * sizeof(uint32_t));
+  o.total = up(o.recs + npts * sizeof(float4));
+  return o;
+}
+
+// tile edge: the largest candidate whose LDS block leaves room for two workgroups per CU
+static void pick_tile(const BwdArgs &a, int &ty, int &tx) {
+  const int cand[][2] = {{16, 16}, {8, 16}, {8, 8}, {4, 8}, {4, 4}, {2, 4}, {2, 2}, {1, 1}};
+  if (a.tile_hint > 0) {
+    ty = a.tile_hint / 100; tx = a.tile_hint % 100;
+    if (ty >= 1 && tx >= 1 && ty <= 64 && tx <= 64) return;
+  }
+  for (auto &c : cand) {
+    ty = c[0]; tx = c[1];
+    if ((size_t)tile_lds_layout(ty, tx, a.C, a.D).total * 4 <= 79 * 1024) return;
+  }
+}
+
+size_t binned_backward_workspace_bytes(const BwdArgs &a, int dtype) {
+  if (dtype == DFA3D_F64) return 0;
+  if ((size_t)a.B * a.Q * a.M * a.L * a.P >= (1ull << 31)) return 0;          // point indices and segment offsets are 32-bit
+  if ((size_t)a.Q * a.M * a.C * 4 >= (size_t)kMaxSliceBytes) return 0;         // grad_out rows are buffer-addressed per batch element
+  int ty = 1, tx = 1;
+  pick_tile(a, ty, tx);
+  if ((size_t)tile_lds_layout(ty, tx, a.C, a.D).total * 4 > 150 * 1024) return 0;   // rows too long for LDS tiles
+  return bin_layout(a, ty, tx).total;
+}
+
+template <typename T, int VEC, int LPR>
+static hipError_t launch_tile_cfg(const BwdArgs &a, const BinWorkspace &ws, int ty, int tx, int block,
+                                  hipStream_t stream) {
+  const size_t lds = (size_t)tile_lds_layout(ty, tx, a.C, a.D).total * 4;
+  auto kern = tile_backward_kernel<T, VEC, LPR>;
+  static thread_local size_t lds_set = 0;
+  if (lds > 64 * 1024 && lds > lds_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    lds_set = lds;
+  }
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) == hipSuccess) hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  const size_t per_cu = lds > 0 ? (160 * 1024) / lds : 8;
+  int wg_per_cu = (int)(per_cu < 1 ? 1 : per_cu > 8 ? 8 : per_cu);
+  const int by_waves = 32 / (block / kWave);
+  if (wg_per_cu > by_waves) wg_per_cu = by_waves < 1 ? 1 : by_waves;
+  const int grid = cus * wg_per_cu;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(block), lds, stream, ws, (const T *)a.value, (const T *)a.dist,
+                     (const float *)a.loc, (const float *)a.attn, (const T *)a.grad_out, (const T *)a.grad_score_in,
+                     (float *)a.grad_value, (float *)a.grad_dist, (float *)a.grad_loc, (float *)a.grad_attn, a.B, a.S,
+                     a.M, a.C, a.D, a.L, a.Q, a.P, a.diag);
+  return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_tile_typed(const BwdArgs &a, const BinWorkspace &ws, int ty, int tx, int block,
+                                    hipStream_t stream) {
+  const RowTiling rt = pick_row_tiling(a.C, (int)sizeof(T), a.vec_hint);
+#define DFA3D_CASE(V, R) \
+  if (rt.vec == V && rt.lpr == R) return launch_tile_cfg<T, V, R>(a, ws, ty, tx, block, stream);
+  DFA3D_ROW_TILINGS(DFA3D_CASE)
+#undef DFA3D_CASE
+  return hipErrorInvalidValue;
+}
+
+// Returns hipErrorNotSupported when the binned path does not apply (caller falls back to the
+// direct kernel).  Needs the fused form (dist given), float or bfloat16 storage, 3-component
+// locations and gradients.
+hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, size_t workspace_bytes,
+                                  hipStream_t stream) {
+  if (a.dist == nullptr || dtype == DFA3D_F64 || a.loc_stride != 3 || a.grad_loc_stride != 3 || a.shape_stride != 3)
+    return hipErrorNotSupported;
+  const size_t need = binned_backward_workspace_bytes(a, dtype);
+  if (need == 0 || workspace == nullptr || workspace_bytes < need || ((uintptr_t)workspace & 255) != 0)
+    return hipErrorNotSupported;
+  const int block = a.block_hint == 256 ? 256 : 512;
+  int ty = 1, tx = 1;
+  pick_tile(a, ty, tx);
+  const BinLayout lay = bin_layout(a, ty, tx);
+  char *base = static_cast<char *>(workspace);
+  BinWorkspace ws;
+  ws.plan = reinterpret_cast<BinPlan *>(base + lay.plan);
+  ws.queues = reinterpret_cast<int *>(base + lay.queues);
+  ws.counts = reinterpret_cast<int *>(base + lay.counts);
+  ws.cursor = reinterpret_cast<int *>(base + lay.cursor);
+  ws.chunk_end = reinterpret_cast<int *>(base + lay.chunk_end);
+  ws.entries = reinterpret_cast<uint32_t *>(base + lay.entries);
+  ws.recs = reinterpret_cast<float4 *>(base + lay.recs);
+  const int mb = max_bins_per_bm(a.S, a.L, ty, tx);
+
+  hipLaunchKernelGGL(plan_and_clear_kernel, dim3(64), dim3(256), 0, stream, ws, a.shapes, a.level_start, a.L, a.S,
+                     a.D, a.B, a.M, ty, tx, a.chunk_hint > 0 ? a.chunk_hint : 1024, mb);
+  const int q_blocks = (a.Q + kBinQueries - 1) / kBinQueries;
+  const long long blocks = (long long)a.B * a.M * q_blocks;
+  if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
+  const int hist_cap = mb < kHistCap ? mb : kHistCap;
+  hipLaunchKernelGGL(bin_points_kernel<0>, dim3((unsigned)blocks), dim3(256), (size_t)hist_cap * 4, stream, ws,
+                     (const float *)a.loc, (const float *)a.attn, (float *)a.grad_loc, (float *)a.grad_attn, a.B, a.M, a.L,
+                     a.Q, a.P, q_blocks, hist_cap);
+  hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(1024), 0, stream, ws);
+  hipLaunchKernelGGL(bin_points_kernel<1>, dim3((unsigned)blocks), dim3(256), (size_t)hist_cap * 8, stream, ws,
+                     (const float *)a.loc, (const float *)a.attn, (float *)a.grad_loc, (float *)a.grad_attn, a.B, a.M, a.L,
+                     a.Q, a.P, q_blocks, hist_cap);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  if (dtype == DFA3D_F32) return launch_tile_typed<float>(a, ws, ty, tx, block, stream);
+  return launch_tile_typed<__hip_bfloat16>(a, ws, ty, tx, block, stream);
+}
+
+}  // namespace dfa3d

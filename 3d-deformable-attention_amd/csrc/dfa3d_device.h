@@ -238,6 +238,7 @@ template <typename A> __device__ __forceinline__ int floor_index(A x) { return (
 template <typename A> struct Point2D {
   A lh, lw, hh, hw;      // fractional parts and complements along h and w
   int key[4];            // key index (level start + h*W + w) of slots LT,RT,RB,LB; -1 outside the map
+  int h0, w0;            // floor of the pixel coordinates (meaningful when `inside`)
   bool inside;           // stage-2 predicate: -1 < h_im < H and -1 < w_im < W
   __device__ __forceinline__ A bil(int k) const {
     return k == 0 ? hh * hw : k == 1 ? hh * lw : k == 2 ? lh * lw : lh * hw;
@@ -250,6 +251,8 @@ __device__ __forceinline__ Point2D<A> locate_2d(A x, A y, int H, int W, int star
   const A h_im = to_pixel(y, H), w_im = to_pixel(x, W);
   g.inside = h_im > -1 && w_im > -1 && h_im < H && w_im < W;
   const int h0 = floor_index(h_im), w0 = floor_index(w_im);
+  g.h0 = h0;
+  g.w0 = w0;
   g.lh = h_im - h0;
   g.lw = w_im - w0;
   g.hh = 1 - g.lh;

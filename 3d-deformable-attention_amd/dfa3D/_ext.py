@@ -281,11 +281,15 @@ def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_leve
     _step(B, im2col_step)
     if grad_output.numel() == 0:
         return
+    code = _lib.dtype_code(value)
+    # scratch for the binned (LDS-accumulating) kernels; 0 bytes means the direct kernel is used
+    ws_bytes = _lib.lib().dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, code)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
     with torch.cuda.device(dev):
         rc = _lib.lib().dfa3d_fused_backward(
             _lib.ptr(value), _lib.ptr(value_dpt_dist), _lib.ptr(value_spatial_shapes),
             _lib.ptr(value_level_start_index), _lib.ptr(sampling_locations), _lib.ptr(attention_weights),
             _lib.ptr(grad_output), _lib.ptr(grad_depth_score), _lib.ptr(grad_value), _lib.ptr(grad_value_dpt_dist),
-            _lib.ptr(grad_sampling_loc), _lib.ptr(grad_attn_weight), B, S, M, C, D, L, Q, P,
-            _lib.dtype_code(value), _lib.stream_of(value))
+            _lib.ptr(grad_sampling_loc), _lib.ptr(grad_attn_weight), _lib.ptr(workspace), ws_bytes,
+            B, S, M, C, D, L, Q, P, code, _lib.stream_of(value))
     _lib.check(rc, "dfa3d_fused_backward")

@@ -99,12 +99,24 @@ int dfa3d_fused_forward(
  * a host synchronisation in the reference).  The depth scores are recomputed from `dist`, not
  * read back.  `grad_score_in` (may be NULL) is an incoming gradient with respect to the `score`
  * output and is chained into grad_dist and the z gradient.  `grad_value` and `grad_dist` are
- * ACCUMULATED into (caller zero-fills); `grad_loc3` and `grad_attn` are overwritten. */
+ * ACCUMULATED into (caller zero-fills); `grad_loc3` and `grad_attn` are overwritten.
+ *
+ * `workspace` (may be NULL) is caller-owned scratch device memory, 256-byte aligned, of at least
+ * dfa3d_fused_backward_workspace_bytes(...) bytes, whose contents need not be preserved or
+ * initialised.  With it (DFA3D_F32 / DFA3D_BF16) the sampling points are first binned by image tile
+ * and every tile of grad_value / grad_dist is accumulated in LDS and written once; without it every
+ * update is a device-memory atomic, which is several times slower.  Results agree up to
+ * floating-point summation order. */
 int dfa3d_fused_backward(
     const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
     const void *loc3, const void *attn, const void *grad_out, const void *grad_score_in,
     void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn,
+    void *workspace, size_t workspace_bytes,
     int B, int S, int M, int C, int D, int L, int Q, int P, int dtype, void *stream);
+
+/* Scratch bytes dfa3d_fused_backward wants for these dimensions; 0 when the binned path does not
+ * apply (DFA3D_F64, rows too long for LDS tiles, more than 2^31 points, invalid dimensions). */
+size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, int L, int Q, int P, int dtype);
 
 /* Message for the last non-zero return on the calling thread ("" if none). */
 const char *dfa3d_last_error(void);
@@ -113,7 +125,10 @@ const char *dfa3d_last_error(void);
  *   "iters"  groups of units each wavefront walks through (default 1)
  *   "vec"    channels per lane in the row gathers: 0 = automatic, 1, 2 or 4
  *   "diag"   measurement aid for the backward kernels: bit 0 drops the grad_value updates,
- *            bit 1 the grad_dist updates (results are then incomplete); default 0 */
+ *            bit 1 the grad_dist updates (results are then incomplete); default 0
+ *   "binned" 0 makes dfa3d_fused_backward ignore its workspace (direct atomic kernel); default 1
+ *   "tile"   binned backward: tile edge in pixels as ty*100+tx, 0 = automatic
+ *   "block"  binned backward: threads per tile workgroup (multiple of 64), 0 = 256 */
 int dfa3d_set_tunable(const char *name, int value);
 
 /* Measurement aid: copies `bytes` (a multiple of 16, 16-byte aligned pointers) from src to dst with
