@@ -39,6 +39,7 @@ std::atomic<int> g_diag{0};
 std::atomic<int> g_tile{0};
 std::atomic<int> g_block{0};
 std::atomic<int> g_chunk{0};
+std::atomic<int> g_stage{0};
 std::atomic<int> g_binned{1};
 int tune_iters() { const int v = g_iters.load(std::memory_order_relaxed); return v < 1 ? 1 : v; }
 int tune_vec() { return g_vec.load(std::memory_order_relaxed); }
@@ -119,9 +120,14 @@ int dfa3d_set_tunable(const char *name, int value) {
     return 0;
   }
   if (!strcmp(name, "chunk")) {
-    if (value != 0 && (value < 64 || value > (1 << 20)))
+    if (value != 0 && (value < 64 || value > (1 << 20)))   // 64 = kMinChunk of the binned backward
       return fail(DFA3D_EINVAL, "dfa3d_set_tunable: chunk must be 0 or in [64, 2^20]");
     g_chunk.store(value, std::memory_order_relaxed);
+    return 0;
+  }
+  if (!strcmp(name, "bwd_stage")) {
+    if (value < 0 || value > 2) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: bwd_stage must be 0, 1 or 2");
+    g_stage.store(value, std::memory_order_relaxed);
     return 0;
   }
   if (!strcmp(name, "binned")) {
@@ -228,6 +234,7 @@ static dfa3d::BwdArgs fused_bwd_args(const void *value, const void *dist, const 
   a.iters = tune_iters(); a.vec_hint = tune_vec(); a.diag = g_diag.load(std::memory_order_relaxed);
   a.tile_hint = g_tile.load(std::memory_order_relaxed); a.block_hint = g_block.load(std::memory_order_relaxed);
   a.chunk_hint = g_chunk.load(std::memory_order_relaxed);
+  a.stage = g_stage.load(std::memory_order_relaxed);
   return a;
 }
 

@@ -46,6 +46,7 @@ struct BinWorkspace {      // device pointers into the caller's workspace
   int *counts;             // points per bin
   int *cursor;             // begin of each bin's segment after the scan, end after the fill
   int *chunk_end;          // inclusive prefix of work items per bin
+  int *item_bin;           // bin of each work item
   uint32_t *entries;       // point indices grouped by bin
   float4 *recs;            // (x, y, z, attention weight) of the same points, same order
 };
@@ -185,7 +186,9 @@ __global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws) {
     const int c = ws.counts[i];
     ws.cursor[i] = run_p;
     run_p += c;
-    run_c += (c + ch - 1) / ch;
+    const int k = (c + ch - 1) / ch;
+    for (int j = 0; j < k; ++j) ws.item_bin[run_c + j] = i;
+    run_c += k;
     ws.chunk_end[i] = run_c;
   }
   if (threadIdx.x == 1023) ws.plan->total_chunks = s_chk[1023];
@@ -300,21 +303,13 @@ __global__ __launch_bounds__(512) void tile_backward_kernel(
   for (int i = tid; i < R * (C + D); i += n_thr) smem[i] = 0;   // gv and gd are adjacent
   TT_DECL
 
-  const int total_bins = p.total_bins, total_chunks = p.total_chunks, CH = p.chunk;
+  const int total_chunks = p.total_chunks, CH = p.chunk;
   for (;;) {
     // ---- next work item: (bin, chunk of its points), in bin order
     __syncthreads();
     if (tid == 0) {
       const int w = atomicAdd(&ws.queues[0], 1);
-      int bin = -1;
-      if (w < total_chunks) {
-        int lo = 0, hi = total_bins - 1;               // first bin whose inclusive chunk prefix exceeds w
-        while (lo < hi) {
-          const int mid = (lo + hi) >> 1;
-          if (ws.chunk_end[mid] > w) hi = mid; else lo = mid + 1;
-        }
-        bin = lo;
-      }
+      const int bin = w < total_chunks ? ws.item_bin[w] : -1;
       s_bin = bin;
       s_item = w;
     }
@@ -542,13 +537,22 @@ __global__ __launch_bounds__(512) void tile_backward_kernel(
     float *gdist_b = grad_dist + (size_t)b * S * M * D;
     const rsrc_t gvalue_r = make_rsrc(gvalue_b, (size_t)S * M * C * sizeof(float));
     const rsrc_t gdist_r = make_rsrc(gdist_b, (size_t)S * M * D * sizeof(float));
+    // Rows 1..TY-1 x 1..TX-1 of the tile belong to no neighbour's halo; when this item holds all the
+    // points of its bin nobody else adds to them, so they are stored instead of added atomically
+    // (grad_value and grad_dist are zero on entry).
+    const bool sole = chunks_here == 1;
     for (int i = tid; i < R * C; i += n_thr) {
       const float val = gv[i];
       if (val != 0) {
         gv[i] = 0;
         const int r = i / C, c = i - r * C;
-        const int y = y0 + r / TW, x = x0 + r % TW;
-        if (y < H && x < W && !(diag & 4)) scatter_add(gvalue_r, gvalue_b, (uint32_t)((((start + y * W + x) * M + m) * C + c) * 4), val);
+        const int ry = r / TW, rx = r % TW;
+        const int y = y0 + ry, x = x0 + rx;
+        if (y < H && x < W && !(diag & 4)) {
+          const uint32_t off = (uint32_t)((((start + y * W + x) * M + m) * C + c) * 4);
+          if (sole && ry >= 1 && ry < TY && rx >= 1 && rx < TX) gvalue_b[off >> 2] = val;
+          else scatter_add(gvalue_r, gvalue_b, off, val);
+        }
       }
     }
     for (int i = tid; i < R * D; i += n_thr) {
@@ -556,8 +560,13 @@ __global__ __launch_bounds__(512) void tile_backward_kernel(
       if (val != 0) {
         gd[i] = 0;
         const int r = i / D, d = i - r * D;
-        const int y = y0 + r / TW, x = x0 + r % TW;
-        if (y < H && x < W && !(diag & 4)) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * M + m) * D + d) * 4), val);
+        const int ry = r / TW, rx = r % TW;
+        const int y = y0 + ry, x = x0 + rx;
+        if (y < H && x < W && !(diag & 4)) {
+          const uint32_t off = (uint32_t)((((start + y * W + x) * M + m) * D + d) * 4);
+          if (sole && ry >= 1 && ry < TY && rx >= 1 && rx < TX) gdist_b[off >> 2] = val;
+          else scatter_add(gdist_r, gdist_b, off, val);
+        }
       }
     }
     TT_MARK(6);
@@ -576,7 +585,8 @@ static int max_bins_per_bm(int S, int L, int ty, int tx) {
   return (int)v;
 }
 
-struct BinLayout { size_t plan, queues, counts, cursor, chunk_end, entries, recs, total; };
+constexpr int kMinChunk = 64;        // smallest accepted points-per-item
+struct BinLayout { size_t plan, queues, counts, cursor, chunk_end, item_bin, entries, recs, total; };
 static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
   BinLayout o;
   const size_t nbins = (size_t)max_bins_per_bm(a.S, a.L, ty, tx) * a.B * a.M;
@@ -587,7 +597,9 @@ static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
   o.counts = up(o.queues + kQueues * sizeof(int));
   o.cursor = up(o.counts + nbins * sizeof(int));
   o.chunk_end = up(o.cursor + nbins * sizeof(int));
-  o.entries = up(o.chunk_end + nbins * sizeof(int));
+  // work items: at most one partial chunk per bin plus the full chunks
+  o.item_bin = up(o.chunk_end + nbins * sizeof(int));
+  o.entries = up(o.item_bin + (nbins + npts / kMinChunk + 1) * sizeof(int));
   o.recs = up(o.entries + npts * sizeof(uint32_t));
   o.total = up(o.recs + npts * sizeof(float4));
   return o;
@@ -674,25 +686,29 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
   ws.counts = reinterpret_cast<int *>(base + lay.counts);
   ws.cursor = reinterpret_cast<int *>(base + lay.cursor);
   ws.chunk_end = reinterpret_cast<int *>(base + lay.chunk_end);
+  ws.item_bin = reinterpret_cast<int *>(base + lay.item_bin);
   ws.entries = reinterpret_cast<uint32_t *>(base + lay.entries);
   ws.recs = reinterpret_cast<float4 *>(base + lay.recs);
   const int mb = max_bins_per_bm(a.S, a.L, ty, tx);
 
-  hipLaunchKernelGGL(plan_and_clear_kernel, dim3(64), dim3(256), 0, stream, ws, a.shapes, a.level_start, a.L, a.S,
-                     a.D, a.B, a.M, ty, tx, a.chunk_hint > 0 ? a.chunk_hint : 1024, mb);
-  const int q_blocks = (a.Q + kBinQueries - 1) / kBinQueries;
-  const long long blocks = (long long)a.B * a.M * q_blocks;
-  if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
-  const int hist_cap = mb < kHistCap ? mb : kHistCap;
-  hipLaunchKernelGGL(bin_points_kernel<0>, dim3((unsigned)blocks), dim3(256), (size_t)hist_cap * 4, stream, ws,
-                     (const float *)a.loc, (const float *)a.attn, (float *)a.grad_loc, (float *)a.grad_attn, a.B, a.M, a.L,
-                     a.Q, a.P, q_blocks, hist_cap);
-  hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(1024), 0, stream, ws);
-  hipLaunchKernelGGL(bin_points_kernel<1>, dim3((unsigned)blocks), dim3(256), (size_t)hist_cap * 8, stream, ws,
-                     (const float *)a.loc, (const float *)a.attn, (float *)a.grad_loc, (float *)a.grad_attn, a.B, a.M, a.L,
-                     a.Q, a.P, q_blocks, hist_cap);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
+  if (a.stage != 2) {
+    hipLaunchKernelGGL(plan_and_clear_kernel, dim3(64), dim3(256), 0, stream, ws, a.shapes, a.level_start, a.L, a.S,
+                       a.D, a.B, a.M, ty, tx, a.chunk_hint > 0 ? a.chunk_hint : 1024, mb);
+    const int q_blocks = (a.Q + kBinQueries - 1) / kBinQueries;
+    const long long blocks = (long long)a.B * a.M * q_blocks;
+    if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
+    const int hist_cap = mb < kHistCap ? mb : kHistCap;
+    hipLaunchKernelGGL(bin_points_kernel<0>, dim3((unsigned)blocks), dim3(256), (size_t)hist_cap * 4, stream, ws,
+                       (const float *)a.loc, (const float *)a.attn, (float *)a.grad_loc, (float *)a.grad_attn, a.B, a.M,
+                       a.L, a.Q, a.P, q_blocks, hist_cap);
+    hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(1024), 0, stream, ws);
+    hipLaunchKernelGGL(bin_points_kernel<1>, dim3((unsigned)blocks), dim3(256), (size_t)hist_cap * 8, stream, ws,
+                       (const float *)a.loc, (const float *)a.attn, (float *)a.grad_loc, (float *)a.grad_attn, a.B, a.M,
+                       a.L, a.Q, a.P, q_blocks, hist_cap);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  if (a.stage == 1) return hipSuccess;
   if (dtype == DFA3D_F32) return launch_tile_typed<float>(a, ws, ty, tx, block, stream);
   return launch_tile_typed<__hip_bfloat16>(a, ws, ty, tx, block, stream);
 }

@@ -9,8 +9,9 @@ BEVFormer-shaped operands already resident in HBM.  Prints ONE JSON line:
 
   metric/value   sampled points (B*Q*M*L*P) per second of forward+backward, whole job
   ms_per_step    forward+backward through autograd (includes its allocations and zero fills)
-  kernels        per-kernel launch durations measured with events on the launch stream, with the
-                 algorithmic GB/s (each operand read once, each result written once) they amount to
+  kernels        launch durations measured with events on the launch stream: the forward kernel, the
+                 backward's binning kernels (as a group) and its tile kernel, with the algorithmic
+                 GB/s (each operand read once, each result written once) they amount to
   roofline       the same for the dominant (longest) kernel, against MI355X's 8 TB/s HBM peak
   cpu_baseline   the scalar C restatement of the operator (oracle/) on the host cores, on a
                  bounded sample of the same workload
@@ -27,8 +28,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (scaled by
-# what the same counters read for a plain copy kernel of known size); see profiles/.
+# HBM-side bytes per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each
+# scaled by what the same counter reads for the library's plain 1 GiB streaming copy (profiles/).
 MEASURED_TRAFFIC_BYTES = {}
 
 
@@ -42,16 +43,14 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain streaming copy of this many MiB (yardstick for profiler HBM counters)")
-    ap.add_argument("--iters", type=int, default=0, help="library tunable 'iters' (0 = default)")
-    ap.add_argument("--vec", type=int, default=-1, help="library tunable 'vec' (-1 = default)")
+    ap.add_argument("--tunable", action="append", default=[], metavar="NAME=VALUE", help="library launch tunable")
     return ap.parse_args()
 
 
 def event_time(fn, reps, prep=None):
-    """Average duration (ms) of fn() on the current stream, bracketed by events per launch."""
+    """Average and minimum duration (ms) of fn() on the current stream, one event pair per call."""
     import torch
-    total = 0.0
-    best = float("inf")
+    total, best = 0.0, float("inf")
     for _ in range(reps):
         if prep is not None:
             prep()
@@ -107,11 +106,10 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP kernels are the product and there is no fallback", file=sys.stderr)
         sys.exit(3)
-    _lib.lib()
-    if a.iters > 0:
-        _lib.set_tunable("iters", a.iters)
-    if a.vec >= 0:
-        _lib.set_tunable("vec", a.vec)
+    L_ = _lib.lib()
+    for t in a.tunable:
+        name, val = t.split("=")
+        _lib.set_tunable(name, int(val))
 
     bf16 = a.workload.endswith("_bf16")
     wname = "base_peaky" if a.workload == "base_bf16" else a.workload
@@ -126,16 +124,13 @@ def main():
     loc, attn = inp["sampling_locations"], inp["attention_weights"]
     e_v = 2 if bf16 else 4
     fwd_bytes, bwd_bytes = w.forward_bytes(e_v, e_v), w.backward_bytes(e_v, e_v)
-    # the fused backward recomputes the depth scores instead of reading the saved ones
-    bwd_bytes_touched = bwd_bytes - 4 * e_v * w.points
 
     if a.calibration_copy_mib > 0:
         n = a.calibration_copy_mib << 20
         src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
         for _ in range(2):
-            _lib.check(_lib.lib().dfa3d_stream_copy(_lib.ptr(dst), _lib.ptr(src), n, _lib.stream_of(src)),
-                       "dfa3d_stream_copy")
+            _lib.check(L_.dfa3d_stream_copy(_lib.ptr(dst), _lib.ptr(src), n, _lib.stream_of(src)), "dfa3d_stream_copy")
         torch.cuda.synchronize()
         del src, dst
 
@@ -165,35 +160,61 @@ def main():
     torch.cuda.synchronize()
     fwd_api_ms = (time.perf_counter() - t0) * 1e3 / a.steps
 
-    # ---- per-kernel durations: one launch between two events on the launch stream ----
-    aux = torch.float32
-    gv = torch.zeros(value.shape, dtype=aux, device=dev)
-    gd = torch.zeros(dist.shape, dtype=aux, device=dev)
+    # ---- per-kernel durations: launches bracketed by events on the launch stream ----
+    B, S, M, C = value.shape
+    D = dist.shape[3]
+    _, Q, _, L, P, _ = loc.shape
+    code = _lib.dtype_code(value)
+    gv = torch.zeros(value.shape, dtype=torch.float32, device=dev)
+    gd = torch.zeros(dist.shape, dtype=torch.float32, device=dev)
     gl = torch.empty_like(loc)
     ga = torch.empty_like(attn)
     vd, dd, ld, ad = value.detach(), dist.detach(), loc.detach(), attn.detach()
-    fwd_ms, fwd_best = event_time(lambda: _ext.dfa3d_fused_forward(vd, dd, shapes, lsi, ld, ad, 64), a.kernel_reps)
+    ws_bytes = L_.dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, code)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    stream = _lib.stream_of(value)
+
+    def backward_call():
+        _lib.check(L_.dfa3d_fused_backward(
+            _lib.ptr(vd), _lib.ptr(dd), _lib.ptr(shapes), _lib.ptr(lsi), _lib.ptr(ld), _lib.ptr(ad), _lib.ptr(go), None,
+            _lib.ptr(gv), _lib.ptr(gd), _lib.ptr(gl), _lib.ptr(ga), _lib.ptr(ws) if ws_bytes else None, ws_bytes,
+            B, S, M, C, D, L, Q, P, code, stream), "dfa3d_fused_backward")
 
     def zero():
         gv.zero_()
         gd.zero_()
 
-    bwd_ms, bwd_best = event_time(
-        lambda: _ext.dfa3d_fused_backward(vd, dd, shapes, lsi, ld, ad, go, None, gv, gd, gl, ga, 64),
-        a.kernel_reps, prep=zero)
+    fwd_ms, fwd_best = event_time(lambda: _ext.dfa3d_fused_forward(vd, dd, shapes, lsi, ld, ad, 64), a.kernel_reps)
+    bwd_all_ms, bwd_all_best = event_time(backward_call, a.kernel_reps, prep=zero)
     fill_ms, _ = event_time(zero, a.kernel_reps)
 
-    def kernel_entry(name, ms, best, nbytes):
+    def entry(name, ms, best, nbytes):
         gbs = nbytes / (ms * 1e-3) / 1e9
-        return {"kernel": name, "avg_ms": round(ms, 4), "min_ms": round(best, 4),
-                "algorithmic_bytes": nbytes, "achieved_gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+        return {"kernel": name, "avg_ms": round(ms, 4), "min_ms": round(best, 4), "algorithmic_bytes": nbytes,
+                "achieved_gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
                 "points_per_s": w.points / (ms * 1e-3)}
 
-    kernels = {
-        "forward": kernel_entry("fwd_attention_kernel (fused depth score + attention)", fwd_ms, fwd_best, fwd_bytes),
-        "backward": kernel_entry("bwd_attention_kernel (fused)", bwd_ms, bwd_best, bwd_bytes),
-    }
-    dom = "backward" if bwd_ms >= fwd_ms else "forward"
+    kernels = {"forward": entry("fwd_attention_kernel (depth score + attention, one launch)", fwd_ms, fwd_best, fwd_bytes)}
+    if ws_bytes:
+        # binning kernels alone, then the tile kernel alone on the workspace they prepared
+        _lib.set_tunable("bwd_stage", 1)
+        bin_ms, bin_best = event_time(backward_call, a.kernel_reps)
+
+        def prepare_tile():
+            zero()
+            _lib.set_tunable("bwd_stage", 1)
+            backward_call()
+            _lib.set_tunable("bwd_stage", 2)
+
+        tile_ms, tile_best = event_time(backward_call, a.kernel_reps, prep=prepare_tile)
+        _lib.set_tunable("bwd_stage", 0)
+        kernels["backward_tile"] = entry("tile_backward_kernel (all gradients, one launch)", tile_ms, tile_best, bwd_bytes)
+        kernels["backward_binning"] = {"kernel": "plan_and_clear + bin_points<0> + bin_scan + bin_points<1> (4 launches)",
+                                       "avg_ms": round(bin_ms, 4), "min_ms": round(bin_best, 4)}
+        dom = "backward_tile" if tile_ms >= fwd_ms else "forward"
+    else:
+        kernels["backward_direct"] = entry("bwd_attention_kernel (device-memory atomics)", bwd_all_ms, bwd_all_best, bwd_bytes)
+        dom = "backward_direct" if bwd_all_ms >= fwd_ms else "forward"
     k = kernels[dom]
     roofline = {"bound": "hbm", "kernel": k["kernel"], "achieved": k["achieved_gbs"], "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": k["frac_of_hbm_peak"], "traffic": MEASURED_TRAFFIC_BYTES.get((a.workload, dom))}
@@ -209,10 +230,10 @@ def main():
         "config": {"workload": f"{a.workload}: B={w.B} Q={w.Q} M={w.M} C={w.C} L={w.L} "
                                f"levels={'/'.join(f'{h}x{x}' for h, x in w.levels)} D={w.D} P={w.P} "
                                f"({w.points} sampled points), one-stage Function forward+backward"},
-        "fwd_ms": round(fwd_api_ms, 4), "fwd_kernel_ms": round(fwd_ms, 4), "bwd_kernel_ms": round(bwd_ms, 4),
-        "grad_zero_fill_ms": round(fill_ms, 4),
+        "fwd_ms": round(fwd_api_ms, 4), "fwd_kernel_ms": round(fwd_ms, 4),
+        "bwd_launches_ms": round(bwd_all_ms, 4), "grad_zero_fill_ms": round(fill_ms, 4),
+        "fwd_points_per_s": w.points / (fwd_api_ms * 1e-3),
         "fwd_frac_of_hbm_peak": kernels["forward"]["frac_of_hbm_peak"],
-        "bwd_bytes_actually_touched": bwd_bytes_touched,
         "kernels": kernels,
         "roofline": roofline,
     }

@@ -128,7 +128,10 @@ const char *dfa3d_last_error(void);
  *            bit 1 the grad_dist updates (results are then incomplete); default 0
  *   "binned" 0 makes dfa3d_fused_backward ignore its workspace (direct atomic kernel); default 1
  *   "tile"   binned backward: tile edge in pixels as ty*100+tx, 0 = automatic
- *   "block"  binned backward: threads per tile workgroup (multiple of 64), 0 = 256 */
+ *   "block"  binned backward: threads per tile workgroup, 256 or 0/512
+ *   "chunk"  binned backward: points of one tile handled by one work item, 0 = 1024
+ *   "bwd_stage" measurement aid for the binned backward: 0 = every kernel, 1 = the binning kernels
+ *            only, 2 = the tile kernel only (on a workspace a stage-1 call has just prepared) */
 int dfa3d_set_tunable(const char *name, int value);
 
 /* Measurement aid: copies `bytes` (a multiple of 16, 16-byte aligned pointers) from src to dst with
