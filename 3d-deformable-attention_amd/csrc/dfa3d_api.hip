@@ -40,6 +40,7 @@ std::atomic<int> g_tile{0};
 std::atomic<int> g_block{0};
 std::atomic<int> g_chunk{0};
 std::atomic<int> g_stage{0};
+std::atomic<int> g_pass{0};
 std::atomic<int> g_binned{1};
 int tune_iters() { const int v = g_iters.load(std::memory_order_relaxed); return v < 1 ? 1 : v; }
 int tune_vec() { return g_vec.load(std::memory_order_relaxed); }
@@ -123,6 +124,11 @@ int dfa3d_set_tunable(const char *name, int value) {
     if (value != 0 && (value < 64 || value > (1 << 20)))   // 64 = kMinChunk of the binned backward
       return fail(DFA3D_EINVAL, "dfa3d_set_tunable: chunk must be 0 or in [64, 2^20]");
     g_chunk.store(value, std::memory_order_relaxed);
+    return 0;
+  }
+  if (!strcmp(name, "pass")) {
+    if (value != 0 && value != 128 && value != 256) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: pass must be 0, 128 or 256");
+    g_pass.store(value, std::memory_order_relaxed);
     return 0;
   }
   if (!strcmp(name, "bwd_stage")) {
@@ -235,6 +241,7 @@ static dfa3d::BwdArgs fused_bwd_args(const void *value, const void *dist, const 
   a.tile_hint = g_tile.load(std::memory_order_relaxed); a.block_hint = g_block.load(std::memory_order_relaxed);
   a.chunk_hint = g_chunk.load(std::memory_order_relaxed);
   a.stage = g_stage.load(std::memory_order_relaxed);
+  a.pass_hint = g_pass.load(std::memory_order_relaxed);
   return a;
 }
 

@@ -286,18 +286,56 @@ template <typename A> __device__ __forceinline__ DepthTap<A> locate_depth(A z, i
   return t;
 }
 
+// Two consecutive elements at byte offset `off` (element-aligned) with ONE load instruction where
+// the hardware allows it: the vector L1 handles roughly one cache line per four clocks whatever the
+// number of bytes used, so the pair costs one line access instead of two.
+template <typename T> struct BufPair;
+template <> struct BufPair<float> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, float &x, float &y) {
+    const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+    x = __uint_as_float(t.x); y = __uint_as_float(t.y);
+  }
+};
+template <> struct BufPair<double> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, double &x, double &y) {
+    const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    x = __hiloint2double((int)t.y, (int)t.x); y = __hiloint2double((int)t.w, (int)t.z);
+  }
+};
+template <> struct BufPair<__hip_bfloat16> {      // a 4-byte load may not sit on a 2-byte boundary: two loads
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, float &x, float &y) {
+    x = BufElem<__hip_bfloat16>::ld(r, off);
+    y = BufElem<__hip_bfloat16>::ld(r, off == kNoRow ? kNoRow : off + 2);
+  }
+};
+
 // Depth scores of the four corners of one point: linear interpolation along depth of the
 // distribution stored at each corner pixel, zero outside the map / outside [0, Dd-1].
 // `dist_r` describes batch element b of dist; lo/hi return the two taps per corner.
 template <typename T, typename A>
 __device__ __forceinline__ void corner_scores(rsrc_t dist_r, const int (&key)[4], const DepthTap<A> &tap, int m, int M,
                                               int D, A (&score)[4], A (&lo)[4], A (&hi)[4]) {
+  if (D >= 2) {
+    // bins (db, db+1) with db clamped into the row always hold both taps that exist
+    const int db = min(max(tap.d0, 0), D - 2);
+    const bool lo_x = tap.lo_ok && tap.d0 == db, lo_y = tap.lo_ok && tap.d0 == db + 1;
+    const bool hi_x = tap.hi_ok && tap.d0 + 1 == db, hi_y = tap.hi_ok && tap.d0 + 1 == db + 1;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const uint32_t row = (uint32_t)(((key[k] * M + m) * D + tap.d0) * (int)sizeof(T));
-    const bool on = key[k] >= 0;
-    lo[k] = BufElem<T>::ld(dist_r, (on && tap.lo_ok) ? row : kNoRow);
-    hi[k] = BufElem<T>::ld(dist_r, (on && tap.hi_ok) ? row + (uint32_t)sizeof(T) : kNoRow);
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t row = (uint32_t)(((key[k] * M + m) * D + db) * (int)sizeof(T));
+      A x, y;
+      BufPair<T>::ld(dist_r, (key[k] >= 0 && tap.inside) ? row : kNoRow, x, y);
+      lo[k] = lo_x ? x : lo_y ? y : (A)0;
+      hi[k] = hi_x ? x : hi_y ? y : (A)0;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t row = (uint32_t)(((key[k] * M + m) * D + tap.d0) * (int)sizeof(T));
+      const bool on = key[k] >= 0;
+      lo[k] = BufElem<T>::ld(dist_r, (on && tap.lo_ok) ? row : kNoRow);
+      hi[k] = BufElem<T>::ld(dist_r, (on && tap.hi_ok) ? row + (uint32_t)sizeof(T) : kNoRow);
+    }
   }
 #pragma unroll
   for (int k = 0; k < 4; ++k) score[k] = lo[k] * tap.hd + hi[k] * tap.ld;

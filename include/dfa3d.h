@@ -129,6 +129,7 @@ const char *dfa3d_last_error(void);
  *   "binned" 0 makes dfa3d_fused_backward ignore its workspace (direct atomic kernel); default 1
  *   "tile"   binned backward: tile edge in pixels as ty*100+tx, 0 = automatic
  *   "block"  binned backward: threads per tile workgroup, 256 or 0/512
+ *   "pass"   binned backward: points a tile workgroup takes per pass, 128 or 0/256
  *   "chunk"  binned backward: points of one tile handled by one work item, 0 = 1024
  *   "bwd_stage" measurement aid for the binned backward: 0 = every kernel, 1 = the binning kernels
  *            only, 2 = the tile kernel only (on a workspace a stage-1 call has just prepared) */
