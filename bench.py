@@ -30,7 +30,11 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 
 # HBM-side bytes per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each
 # scaled by what the same counter reads for the library's plain 1 GiB streaming copy (profiles/).
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/fwd_attention_and_tile_backward_base_fp32.txt
+    ("base", "forward"): 5.22e9,
+    ("base", "backward_tile"): 5.91e9,
+}
 
 
 def parse():
