@@ -92,7 +92,7 @@ int dfa3d_stream_copy(void *dst, const void *src, size_t bytes, void *stream) {
 }
 
 const char *dfa3d_last_error(void) { return g_err; }
-int dfa3d_abi_version(void) { return 2; }
+int dfa3d_abi_version(void) { return 3; }
 
 int dfa3d_set_tunable(const char *name, int value) {
   if (name == nullptr) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: name is NULL");
@@ -158,14 +158,29 @@ int dfa3d_ms_depth_score_sample_forward(const void *dist, const int64_t *shapes3
   return hip_result(dfa3d::launch_depth_score(a, dtype, (hipStream_t)stream), fn);
 }
 
+size_t dfa3d_ms_depth_score_sample_backward_workspace_bytes(int B, int S, int M, int D, int L, int Q, int P,
+                                                            int dtype) {
+  if (check_dims("dfa3d_ms_depth_score_sample_backward_workspace_bytes", B, S, M, D, L, Q, P, dtype)) return 0;
+  if (!g_binned.load(std::memory_order_relaxed)) return 0;
+  dfa3d::DepthScoreBwdArgs a{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, B, S, M, D, L, Q, P};
+  return dfa3d::binned_depth_score_backward_workspace_bytes(a, dtype, g_tile.load(std::memory_order_relaxed));
+}
+
 int dfa3d_ms_depth_score_sample_backward(const void *dist, const int64_t *shapes3, const int64_t *level_start,
                                          const void *loc3, const void *grad_score, void *grad_dist, void *grad_loc3,
+                                         void *workspace, size_t workspace_bytes,
                                          int B, int S, int M, int D, int L, int Q, int P, int dtype, void *stream) {
   const char *fn = "dfa3d_ms_depth_score_sample_backward";
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
   REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start); REQUIRE_PTR(fn, loc3);
   REQUIRE_PTR(fn, grad_score); REQUIRE_PTR(fn, grad_dist); REQUIRE_PTR(fn, grad_loc3);
   dfa3d::DepthScoreBwdArgs a{dist, shapes3, level_start, loc3, grad_score, grad_dist, grad_loc3, B, S, M, D, L, Q, P};
+  if (workspace != nullptr && g_binned.load(std::memory_order_relaxed)) {
+    const hipError_t e = dfa3d::launch_depth_score_backward_binned(
+        a, dtype, workspace, workspace_bytes, g_tile.load(std::memory_order_relaxed),
+        g_chunk.load(std::memory_order_relaxed), (hipStream_t)stream);
+    if (e != hipErrorNotSupported) return hip_result(e, fn);
+  }
   return hip_result(dfa3d::launch_depth_score_backward(a, dtype, (hipStream_t)stream), fn);
 }
 
@@ -187,10 +202,38 @@ int dfa3d_wms_deform_attn_forward(const void *value, const int64_t *shapes, int 
   return hip_result(dfa3d::launch_forward(a, dtype, (hipStream_t)stream), fn);
 }
 
-int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int shape_stride,
+static dfa3d::BwdArgs wms_bwd_args(const void *value, const int64_t *shapes, int shape_stride,
                                    const int64_t *level_start, const void *loc, int loc_stride, const void *attn,
                                    const void *score, const void *grad_out, void *grad_value, void *grad_loc,
                                    int grad_loc_stride, void *grad_attn, void *grad_score, int B, int S, int M, int C,
+                                   int L, int Q, int P) {
+  dfa3d::BwdArgs a{};
+  a.value = value; a.dist = nullptr; a.shapes = shapes; a.shape_stride = shape_stride; a.level_start = level_start;
+  a.loc = loc; a.loc_stride = loc_stride; a.attn = attn; a.score_in = score; a.grad_out = grad_out;
+  a.grad_score_in = nullptr; a.grad_value = grad_value; a.grad_dist = nullptr; a.grad_loc = grad_loc;
+  a.grad_loc_stride = grad_loc_stride; a.grad_attn = grad_attn; a.grad_score_out = grad_score;
+  a.B = B; a.S = S; a.M = M; a.C = C; a.D = 1; a.L = L; a.Q = Q; a.P = P;
+  a.iters = tune_iters(); a.vec_hint = tune_vec(); a.diag = g_diag.load(std::memory_order_relaxed);
+  a.tile_hint = g_tile.load(std::memory_order_relaxed); a.block_hint = g_block.load(std::memory_order_relaxed);
+  a.chunk_hint = g_chunk.load(std::memory_order_relaxed);
+  a.stage = g_stage.load(std::memory_order_relaxed);
+  a.pass_hint = g_pass.load(std::memory_order_relaxed);
+  return a;
+}
+
+size_t dfa3d_wms_deform_attn_backward_workspace_bytes(int B, int S, int M, int C, int L, int Q, int P, int dtype) {
+  if (check_dims("dfa3d_wms_deform_attn_backward_workspace_bytes", B, S, M, C, L, Q, P, dtype)) return 0;
+  if (!g_binned.load(std::memory_order_relaxed)) return 0;
+  const dfa3d::BwdArgs a = wms_bwd_args(nullptr, nullptr, 2, nullptr, nullptr, 2, nullptr, nullptr, nullptr, nullptr,
+                                        nullptr, 2, nullptr, nullptr, B, S, M, C, L, Q, P);
+  return dfa3d::binned_backward_workspace_bytes(a, 1, dtype);
+}
+
+int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int shape_stride,
+                                   const int64_t *level_start, const void *loc, int loc_stride, const void *attn,
+                                   const void *score, const void *grad_out, void *grad_value, void *grad_loc,
+                                   int grad_loc_stride, void *grad_attn, void *grad_score,
+                                   void *workspace, size_t workspace_bytes, int B, int S, int M, int C,
                                    int L, int Q, int P, int dtype, void *stream) {
   const char *fn = "dfa3d_wms_deform_attn_backward";
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
@@ -200,13 +243,13 @@ int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, shapes); REQUIRE_PTR(fn, level_start); REQUIRE_PTR(fn, loc);
   REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, score); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
   REQUIRE_PTR(fn, grad_loc); REQUIRE_PTR(fn, grad_attn); REQUIRE_PTR(fn, grad_score);
-  dfa3d::BwdArgs a{};
-  a.value = value; a.dist = nullptr; a.shapes = shapes; a.shape_stride = shape_stride; a.level_start = level_start;
-  a.loc = loc; a.loc_stride = loc_stride; a.attn = attn; a.score_in = score; a.grad_out = grad_out;
-  a.grad_score_in = nullptr; a.grad_value = grad_value; a.grad_dist = nullptr; a.grad_loc = grad_loc;
-  a.grad_loc_stride = grad_loc_stride; a.grad_attn = grad_attn; a.grad_score_out = grad_score;
-  a.B = B; a.S = S; a.M = M; a.C = C; a.D = 1; a.L = L; a.Q = Q; a.P = P;
-  a.iters = tune_iters(); a.vec_hint = tune_vec(); a.diag = g_diag.load(std::memory_order_relaxed);
+  const dfa3d::BwdArgs a = wms_bwd_args(value, shapes, shape_stride, level_start, loc, loc_stride, attn, score,
+                                        grad_out, grad_value, grad_loc, grad_loc_stride, grad_attn, grad_score, B, S,
+                                        M, C, L, Q, P);
+  if (workspace != nullptr && g_binned.load(std::memory_order_relaxed)) {
+    const hipError_t e = dfa3d::launch_backward_binned(a, dtype, workspace, workspace_bytes, (hipStream_t)stream);
+    if (e != hipErrorNotSupported) return hip_result(e, fn);
+  }
   return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
 }
 
@@ -251,7 +294,7 @@ size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, i
   if (!g_binned.load(std::memory_order_relaxed)) return 0;
   const dfa3d::BwdArgs a = fused_bwd_args(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
                                           nullptr, nullptr, nullptr, nullptr, B, S, M, C, D, L, Q, P);
-  return dfa3d::binned_backward_workspace_bytes(a, dtype);
+  return dfa3d::binned_backward_workspace_bytes(a, 0, dtype);
 }
 
 int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,

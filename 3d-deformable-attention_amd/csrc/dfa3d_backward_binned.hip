@@ -53,7 +53,8 @@ struct BinWorkspace {      // device pointers into the caller's workspace
 
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void plan_and_clear_kernel(
-    BinWorkspace ws, const int64_t *__restrict__ shapes3, const int64_t *__restrict__ level_start, int L, int S, int D,
+    BinWorkspace ws, const int64_t *__restrict__ shapes, int shape_stride, const int64_t *__restrict__ level_start, int L,
+    int S, int D,
     int B, int M, int ty, int tx, int chunk, int max_bins_per_bm) {
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     BinPlan p;
@@ -62,8 +63,10 @@ __global__ __launch_bounds__(256) void plan_and_clear_kernel(
       int64_t H = 0, W = 0, Dd = 0, st = 0;
       bool ok = false;
       if (l < L) {
-        H = shapes3[l * 3]; W = shapes3[l * 3 + 1]; Dd = shapes3[l * 3 + 2]; st = level_start[l];
-        ok = H > 0 && W > 0 && st >= 0 && H <= S && W <= S && st + H * W <= (int64_t)S && Dd > 0 && Dd <= D;
+        H = shapes[l * shape_stride]; W = shapes[l * shape_stride + 1];
+        Dd = (shape_stride > 2 && D > 0) ? shapes[l * shape_stride + 2] : 1; st = level_start[l];
+        ok = H > 0 && W > 0 && st >= 0 && H <= S && W <= S && st + H * W <= (int64_t)S && Dd > 0 &&
+             (D <= 0 || Dd <= D);
       }
       p.H[l] = ok ? (int)H : 0; p.W[l] = ok ? (int)W : 0; p.Dd[l] = ok ? (int)Dd : 0; p.start[l] = ok ? (int)st : 0;
       const int nx = ok ? ((int)W + tx - 1) / tx : 0, ny = ok ? ((int)H + ty - 1) / ty : 0;
@@ -96,8 +99,9 @@ __device__ __forceinline__ int bin_of(const BinPlan &p, int l, const Point2D<flo
 // MODE 0: count.  MODE 1: fill (needs the scanned cursor).
 template <int MODE>
 __global__ __launch_bounds__(256) void bin_points_kernel(
-    BinWorkspace ws, const float *__restrict__ loc3, const float *__restrict__ attn, float *__restrict__ grad_loc3,
-    float *__restrict__ grad_attn, int B, int M, int L, int Q, int P, int q_blocks, int hist_cap, int diag) {
+    BinWorkspace ws, const float *__restrict__ loc, int loc_stride, const float *__restrict__ attn,
+    float *__restrict__ grad_loc, int gl_stride, float *__restrict__ grad_attn, float *__restrict__ grad_score,
+    int B, int M, int L, int Q, int P, int q_blocks, int hist_cap, int diag) {
   extern __shared__ int s_hist[];          // [0, nb): counts, then for MODE 1 [nb, 2 nb): segment bases
   const BinPlan &p = *ws.plan;
   const int nb = p.bins_per_bm;
@@ -119,15 +123,18 @@ __global__ __launch_bounds__(256) void bin_points_kernel(
   for (int i = threadIdx.x; i < npts; i += blockDim.x) {
     const int qi = i / LP, lp = i - qi * LP, l = lp / P;
     const size_t gp = ((size_t)(b * (size_t)Q + q0 + qi) * M + m) * LP + lp;
-    const Point2D<float> g = locate_2d<float>(loc3[gp * 3], loc3[gp * 3 + 1], p.H[l], p.W[l], p.start[l]);
+    const Point2D<float> g = locate_2d<float>(loc[gp * loc_stride], loc[gp * loc_stride + 1], p.H[l], p.W[l], p.start[l]);
     if (g.inside && p.tiles_x[l] > 0) {
       const int bin = bin_of(p, l, g);
       if (use_lds) atomicAdd(&s_hist[bin], 1);
       else if (MODE == 0) atomicAdd(&gcount[bin], 1);
     } else if (MODE == 1) {
       // skipped by the operator: all its gradients are zero, and no tile will visit it
-      grad_loc3[gp * 3] = 0; grad_loc3[gp * 3 + 1] = 0; grad_loc3[gp * 3 + 2] = 0;
-      grad_attn[gp] = 0;
+      for (int i = 0; i < gl_stride; ++i) grad_loc[gp * gl_stride + i] = 0;
+      if (grad_attn != nullptr) grad_attn[gp] = 0;
+      if (grad_score != nullptr) {
+        for (int k = 0; k < 4; ++k) grad_score[gp * 4 + k] = 0;
+      }
     }
   }
   if (use_lds) {
@@ -147,12 +154,14 @@ __global__ __launch_bounds__(256) void bin_points_kernel(
     for (int i = threadIdx.x; i < npts; i += blockDim.x) {
       const int qi = i / LP, lp = i - qi * LP, l = lp / P;
       const size_t gp = ((size_t)(b * (size_t)Q + q0 + qi) * M + m) * LP + lp;
-      const Point2D<float> g = locate_2d<float>(loc3[gp * 3], loc3[gp * 3 + 1], p.H[l], p.W[l], p.start[l]);
+      const Point2D<float> g = locate_2d<float>(loc[gp * loc_stride], loc[gp * loc_stride + 1], p.H[l], p.W[l], p.start[l]);
       if (g.inside && p.tiles_x[l] > 0) {
         const int bin = bin_of(p, l, g);
         const int slot = use_lds ? s_hist[nb + bin] + atomicAdd(&s_hist[bin], 1) : atomicAdd(&gcursor[bin], 1);
         if (!(diag & 128)) ws.entries[slot] = (uint32_t)gp;
-        if (!(diag & 64)) ws.recs[slot] = make_float4(loc3[gp * 3], loc3[gp * 3 + 1], loc3[gp * 3 + 2], attn[gp]);
+        if (!(diag & 64))
+          ws.recs[slot] = make_float4(loc[gp * loc_stride], loc[gp * loc_stride + 1],
+                                      loc_stride > 2 ? loc[gp * loc_stride + 2] : 0.f, attn != nullptr ? attn[gp] : 0.f);
       }
     }
   }
@@ -293,12 +302,16 @@ template <> struct LdsVec<4> {
 };
 template <int VEC> __device__ __forceinline__ void lds_ld(const float *p, float (&v)[VEC]) { LdsVec<VEC>::ld(p, v); }
 
-template <typename T, int VEC, int LPR>
+// FUSED: both stages (depth scores recomputed from dist, grad_dist and the z gradient produced).
+// !FUSED: stage 2 alone: scores read from score_in, their gradient written to grad_score_out, no
+// depth tile (the launcher passes D = 0), grad_loc has gl_stride components of which x, y are written.
+template <typename T, int VEC, int LPR, bool FUSED>
 __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
-    BinWorkspace ws, const T *__restrict__ value, const T *__restrict__ dist, const float *__restrict__ loc3,
-    const float *__restrict__ attn, const T *__restrict__ grad_out, const T *__restrict__ grad_score_in,
-    float *__restrict__ grad_value, float *__restrict__ grad_dist, float *__restrict__ grad_loc3,
-    float *__restrict__ grad_attn, int B, int S, int M, int C, int D, int L, int Q, int P, int PP, int diag) {
+    BinWorkspace ws, const T *__restrict__ value, const T *__restrict__ dist, const T *__restrict__ score_in,
+    const T *__restrict__ grad_out, const T *__restrict__ grad_score_in,
+    float *__restrict__ grad_value, float *__restrict__ grad_dist, float *__restrict__ grad_loc, int gl_stride,
+    float *__restrict__ grad_attn, float *__restrict__ grad_score_out,
+    int B, int S, int M, int C, int D, int L, int Q, int P, int PP, int diag) {
   constexpr int RPI = kWave / LPR;                  // row groups per wavefront
   extern __shared__ __align__(16) float smem[];
   __shared__ int s_bin, s_item;
@@ -352,7 +365,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
     const int y0 = (tile / p.tiles_x[l]) * TY, x0 = (tile % p.tiles_x[l]) * TX;
 
     const rsrc_t value_r = make_rsrc(value + (size_t)b * S * M * C, (size_t)S * M * C * sizeof(T));
-    const rsrc_t dist_r = make_rsrc(dist + (size_t)b * S * M * D, (size_t)S * M * D * sizeof(T));
+    const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * M * D : nullptr, FUSED ? (size_t)S * M * D * sizeof(T) : 0);
     const rsrc_t go_r = make_rsrc(grad_out + (size_t)b * Q * M * C, (size_t)Q * M * C * sizeof(T));
 
     for (int base = 0; base < n_item; base += PP) {               // uniform over the workgroup
@@ -376,8 +389,14 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const size_t unit = gp / LP;
         a = rec.w;
         g = locate_2d<float>(rec.x, rec.y, H, W, start);
-        tap = locate_depth<float>(rec.z, Dd);
-        corner_scores<T, float>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
+        if (FUSED) {
+          tap = locate_depth<float>(rec.z, Dd);
+          corner_scores<T, float>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
+        } else {
+          const T *si = score_in + gp * 4;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) sc[k] = Elem<T>::ld(si + k);
+        }
         my_goff = (uint32_t)((unit - (size_t)b * Q * M) * C * sizeof(T));
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -532,26 +551,31 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         }
         const float gx = (float)W * a * (g.hh * (s[1] - s[0]) + g.lh * (s[2] - s[3]));
         const float gy = (float)H * a * (g.hw * (s[3] - s[0]) + g.lw * (s[2] - s[1]));
-        if (grad_score_in != nullptr) {
-          const T *gi = grad_score_in + gp * 4;
-#pragma unroll
-          for (int k = 0; k < 4; ++k) gs[k] += Elem<T>::ld(gi + k);
-        }
-        float gz = 0;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          if (tr[k] >= 0 && tap.inside && gs[k] != 0 && !(diag & 2)) {
-            float *dst = gd + tr[k] * D + tap.d0;
-            if (tap.lo_ok) atomicAdd(dst, tap.hd * gs[k]);
-            if (tap.hi_ok) atomicAdd(dst + 1, tap.ld * gs[k]);
-          }
-          gz += (g.key[k] >= 0 && tap.inside) ? gs[k] * (hi[k] - lo[k]) : 0.f;
-        }
-        // 16 scattered bytes per point: measured cheaper than writing them in bin order and
-        // un-sorting in a separate pass (0.14 ms against 0.25 ms at the BEVFormer-base shape)
-        float *gl = grad_loc3 + gp * 3;
-        gl[0] = gx; gl[1] = gy; gl[2] = gz * (float)Dd;
+        float *gl = grad_loc + gp * gl_stride;
+        gl[0] = gx; gl[1] = gy;
         grad_attn[gp] = ga;
+        if (FUSED) {
+          if (grad_score_in != nullptr) {
+            const T *gi = grad_score_in + gp * 4;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) gs[k] += Elem<T>::ld(gi + k);
+          }
+          float gz = 0;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            if (tr[k] >= 0 && tap.inside && gs[k] != 0 && !(diag & 2)) {
+              float *dst = gd + tr[k] * D + tap.d0;
+              if (tap.lo_ok) atomicAdd(dst, tap.hd * gs[k]);
+              if (tap.hi_ok) atomicAdd(dst + 1, tap.ld * gs[k]);
+            }
+            gz += (g.key[k] >= 0 && tap.inside) ? gs[k] * (hi[k] - lo[k]) : 0.f;
+          }
+          gl[2] = gz * (float)Dd;
+        } else {
+          float *go4 = grad_score_out + gp * 4;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) go4[k] = gs[k];
+        }
       }
       __syncthreads();                                   // before the next pass reuses the scratch arrays
       TT_MARK(5);
@@ -559,9 +583,9 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
 
     // ---------------- flush the tile (and leave it zeroed for the next item) ----------------
     float *gvalue_b = grad_value + (size_t)b * S * M * C;
-    float *gdist_b = grad_dist + (size_t)b * S * M * D;
+    float *gdist_b = FUSED ? grad_dist + (size_t)b * S * M * D : nullptr;
     const rsrc_t gvalue_r = make_rsrc(gvalue_b, (size_t)S * M * C * sizeof(float));
-    const rsrc_t gdist_r = make_rsrc(gdist_b, (size_t)S * M * D * sizeof(float));
+    const rsrc_t gdist_r = make_rsrc(gdist_b, FUSED ? (size_t)S * M * D * sizeof(float) : 0);
     // Rows 1..TY-1 x 1..TX-1 of the tile belong to no neighbour's halo; when this item holds all the
     // points of its bin nobody else adds to them, so they are stored instead of added atomically
     // (grad_value and grad_dist are zero on entry).
@@ -636,6 +660,89 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
+// Stage-1 backward alone on the same bins: the gradient with respect to the four depth scores of
+// each point is given; grad_dist is accumulated in an LDS tile, the z gradient written per point.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void tile_depth_backward_kernel(
+    BinWorkspace ws, const T *__restrict__ dist, const T *__restrict__ grad_score, float *__restrict__ grad_dist,
+    float *__restrict__ grad_loc3, int B, int S, int M, int D, int L, int Q, int P) {
+  extern __shared__ __align__(16) float smem[];
+  __shared__ int s_bin, s_item;
+  const BinPlan &p = *ws.plan;
+  const int nb = p.bins_per_bm;
+  if (nb == 0) return;
+  const int TY = p.ty, TX = p.tx, TW = TX + 1, R = (TY + 1) * TW;
+  const int tid = threadIdx.x, n_thr = blockDim.x;
+  float *gd = smem;
+  for (int i = tid; i < R * D; i += n_thr) gd[i] = 0;
+  const int total_chunks = p.total_chunks, CH = p.chunk;
+  for (;;) {
+    __syncthreads();
+    if (tid == 0) {
+      const int w = atomicAdd(&ws.queues[0], 1);
+      s_bin = w < total_chunks ? ws.item_bin[w] : -1;
+      s_item = w;
+    }
+    __syncthreads();
+    const int bin = s_bin;
+    if (bin < 0) break;                                   // queue drained: every wave leaves
+    const int n_bin = ws.counts[bin];
+    const int chunks_here = (n_bin + CH - 1) / CH;
+    const int chunk_id = s_item - (ws.chunk_end[bin] - chunks_here);
+    const int first = chunk_id * CH;
+    const int n_item = min(CH, n_bin - first);
+    const int seg = ws.cursor[bin] - n_bin + first;
+    const int bm = bin / nb, local = bin - bm * nb;
+    const int b = bm / M, m = bm - b * M;
+    int l = 0;
+    while (l + 1 < L && local >= p.level_base[l + 1]) ++l;
+    const int tile = local - p.level_base[l];
+    const int H = p.H[l], W = p.W[l], Dd = p.Dd[l], start = p.start[l];
+    const int y0 = (tile / p.tiles_x[l]) * TY, x0 = (tile % p.tiles_x[l]) * TX;
+    const rsrc_t dist_r = make_rsrc(dist + (size_t)b * S * M * D, (size_t)S * M * D * sizeof(T));
+
+    for (int i = tid; i < n_item; i += n_thr) {
+      const size_t gp = ws.entries[seg + i];
+      const float4 rec = ws.recs[seg + i];
+      const Point2D<float> g = locate_2d<float>(rec.x, rec.y, H, W, start);
+      const DepthTap<float> tap = locate_depth<float>(rec.z, Dd);
+      float sc[4], lo[4], hi[4];
+      corner_scores<T, float>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
+      const T *gi = grad_score + gp * 4;
+      float gz = 0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (g.key[k] >= 0 && tap.inside) {
+          const float gk = Elem<T>::ld(gi + k);
+          const int ry = g.h0 + (k >= 2 ? 1 : 0) - y0, rx = g.w0 + ((k == 1 || k == 2) ? 1 : 0) - x0;
+          if (ry >= 0 && ry <= TY && rx >= 0 && rx <= TX && gk != 0) {
+            float *dst = gd + (ry * TW + rx) * D + tap.d0;
+            if (tap.lo_ok) atomicAdd(dst, tap.hd * gk);
+            if (tap.hi_ok) atomicAdd(dst + 1, tap.ld * gk);
+          }
+          gz += gk * (hi[k] - lo[k]);
+        }
+      }
+      float *gl = grad_loc3 + gp * 3;
+      gl[0] = 0; gl[1] = 0; gl[2] = gz * (float)Dd;
+    }
+    __syncthreads();
+    float *gdist_b = grad_dist + (size_t)b * S * M * D;
+    const rsrc_t gdist_r = make_rsrc(gdist_b, (size_t)S * M * D * sizeof(float));
+    for (int i = tid; i < R * D; i += n_thr) {
+      const float val = gd[i];
+      if (val != 0) {
+        gd[i] = 0;
+        const int r = i / D, d = i - r * D;
+        const int y = y0 + r / TW, x = x0 + r % TW;
+        if (y < H && x < W) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * M + m) * D + d) * 4), val);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
 static int max_bins_per_bm(int S, int L, int ty, int tx) {
@@ -665,63 +772,89 @@ static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
   return o;
 }
 
-// Launch shape of the tile kernel: tile edge, threads per workgroup, points per pass.
+// Launch shape of the tile kernels: tile edge, threads per workgroup, points per pass.
 struct TileConfig { int ty, tx, block, pp; size_t lds; };
+
+// kind 0: both stages, 1: stage 2 alone (no depth tile), 2: stage 1 alone (depth tile only)
+static size_t tile_lds_bytes(int kind, int ty, int tx, int C, int D, int pp) {
+  if (kind == 2) return (size_t)(ty + 1) * (tx + 1) * D * 4;
+  return (size_t)tile_lds_layout(ty, tx, C, kind == 1 ? 0 : D, pp).total * 4;
+}
 
 // Defaults: 512 threads taking 256 points per pass, and the largest tile whose LDS block still
 // lets two workgroups share a CU.
-static TileConfig pick_tile_config(const BwdArgs &a) {
+static TileConfig pick_tile_config(int kind, int C, int D, int tile_hint, int block_hint, int pass_hint) {
   TileConfig c;
-  c.block = a.block_hint == 256 ? 256 : 512;
-  c.pp = (a.pass_hint == 128 || a.pass_hint == 256) ? a.pass_hint : 256;
+  c.block = kind == 2 ? 256 : (block_hint == 256 ? 256 : 512);
+  c.pp = (pass_hint == 128 || pass_hint == 256) ? pass_hint : 256;
   if (c.pp > c.block) c.pp = c.block;
   const int cand[][2] = {{16, 16}, {8, 16}, {8, 8}, {4, 8}, {4, 4}, {2, 4}, {2, 2}, {1, 1}};
   c.ty = c.tx = 1;
-  const int hy = a.tile_hint / 100, hx = a.tile_hint % 100;
-  if (a.tile_hint > 0 && hy >= 1 && hx >= 1 && hy <= 64 && hx <= 64) {
+  const int hy = tile_hint / 100, hx = tile_hint % 100;
+  if (tile_hint > 0 && hy >= 1 && hx >= 1 && hy <= 64 && hx <= 64) {
     c.ty = hy; c.tx = hx;
   } else {
+    const size_t budget = kind == 2 ? 40 * 1024 : 79 * 1024;
     for (auto &t : cand) {
       c.ty = t[0]; c.tx = t[1];
-      if ((size_t)tile_lds_layout(c.ty, c.tx, a.C, a.D, c.pp).total * 4 <= 79 * 1024) break;
+      if (tile_lds_bytes(kind, c.ty, c.tx, C, D, c.pp) <= budget) break;
     }
   }
-  c.lds = (size_t)tile_lds_layout(c.ty, c.tx, a.C, a.D, c.pp).total * 4;
+  c.lds = tile_lds_bytes(kind, c.ty, c.tx, C, D, c.pp);
   return c;
 }
 
-size_t binned_backward_workspace_bytes(const BwdArgs &a, int dtype) {
+static int bwd_kind(const BwdArgs &a) { return a.dist != nullptr ? 0 : 1; }
+static TileConfig tile_config_of(const BwdArgs &a, int kind) {
+  return pick_tile_config(kind, a.C, a.D, a.tile_hint, a.block_hint, a.pass_hint);
+}
+
+static size_t workspace_bytes_for(const BwdArgs &a, int kind, int dtype) {
   if (dtype == DFA3D_F64) return 0;
   if ((size_t)a.B * a.Q * a.M * a.L * a.P >= (1ull << 31)) return 0;          // point indices and segment offsets are 32-bit
-  if ((size_t)a.Q * a.M * a.C * 4 >= (size_t)kMaxSliceBytes) return 0;         // grad_out rows are buffer-addressed per batch element
-  const TileConfig c = pick_tile_config(a);
+  if (kind != 2 && (size_t)a.Q * a.M * a.C * 4 >= (size_t)kMaxSliceBytes) return 0;   // grad_out rows are buffer-addressed per batch element
+  const TileConfig c = tile_config_of(a, kind);
   if (c.lds > 150 * 1024) return 0;                                            // rows too long for LDS tiles
   return bin_layout(a, c.ty, c.tx).total;
 }
 
-template <typename T, int VEC, int LPR>
-static hipError_t launch_tile_cfg(const BwdArgs &a, const BinWorkspace &ws, const TileConfig &c, hipStream_t stream) {
-  const size_t lds = c.lds;
-  const int block = c.block;
-  auto kern = tile_backward_kernel<T, VEC, LPR>;
-  static thread_local size_t lds_set = 0;
-  if (lds > 64 * 1024 && lds > lds_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    lds_set = lds;
-  }
+// kind as in tile_lds_bytes; `a.dist != nullptr` is not consulted here, so dimension-only queries work
+size_t binned_backward_workspace_bytes(const BwdArgs &a, int kind, int dtype) { return workspace_bytes_for(a, kind, dtype); }
+
+static int tile_grid(size_t lds, int block) {
   int dev = 0, cus = 256;
-  if (hipGetDevice(&dev) == hipSuccess) hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+    cus = 256;
   const size_t per_cu = lds > 0 ? (160 * 1024) / lds : 8;
   int wg_per_cu = (int)(per_cu < 1 ? 1 : per_cu > 8 ? 8 : per_cu);
   const int by_waves = 32 / (block / kWave);
   if (wg_per_cu > by_waves) wg_per_cu = by_waves < 1 ? 1 : by_waves;
-  const int grid = cus * wg_per_cu;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(block), lds, stream, ws, (const T *)a.value, (const T *)a.dist,
-                     (const float *)a.loc, (const float *)a.attn, (const T *)a.grad_out, (const T *)a.grad_score_in,
-                     (float *)a.grad_value, (float *)a.grad_dist, (float *)a.grad_loc, (float *)a.grad_attn, a.B, a.S,
-                     a.M, a.C, a.D, a.L, a.Q, a.P, c.pp, a.diag);
+  return cus * wg_per_cu;
+}
+
+template <typename K> static hipError_t allow_lds(K kern, size_t lds) {
+  if (lds <= 64 * 1024) return hipSuccess;
+  return hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+}
+
+template <typename T, int VEC, int LPR>
+static hipError_t launch_tile_cfg(const BwdArgs &a, const BinWorkspace &ws, const TileConfig &c, hipStream_t stream) {
+  const int grid = tile_grid(c.lds, c.block);
+  if (a.dist != nullptr) {
+    auto kern = tile_backward_kernel<T, VEC, LPR, true>;
+    if (hipError_t e = allow_lds(kern, c.lds)) return e;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(c.block), c.lds, stream, ws, (const T *)a.value, (const T *)a.dist,
+                       (const T *)nullptr, (const T *)a.grad_out, (const T *)a.grad_score_in, (float *)a.grad_value,
+                       (float *)a.grad_dist, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
+                       (float *)nullptr, a.B, a.S, a.M, a.C, a.D, a.L, a.Q, a.P, c.pp, a.diag);
+  } else {
+    auto kern = tile_backward_kernel<T, VEC, LPR, false>;
+    if (hipError_t e = allow_lds(kern, c.lds)) return e;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(c.block), c.lds, stream, ws, (const T *)a.value, (const T *)nullptr,
+                       (const T *)a.score_in, (const T *)a.grad_out, (const T *)nullptr, (float *)a.grad_value,
+                       (float *)nullptr, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
+                       (float *)a.grad_score_out, a.B, a.S, a.M, a.C, 0, a.L, a.Q, a.P, c.pp, a.diag);
+  }
   return hipGetLastError();
 }
 
@@ -735,19 +868,7 @@ static hipError_t launch_tile_typed(const BwdArgs &a, const BinWorkspace &ws, co
   return hipErrorInvalidValue;
 }
 
-// Returns hipErrorNotSupported when the binned path does not apply (caller falls back to the
-// direct kernel).  Needs the fused form (dist given), float or bfloat16 storage, 3-component
-// locations and gradients.
-hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, size_t workspace_bytes,
-                                  hipStream_t stream) {
-  if (a.dist == nullptr || dtype == DFA3D_F64 || a.loc_stride != 3 || a.grad_loc_stride != 3 || a.shape_stride != 3)
-    return hipErrorNotSupported;
-  const size_t need = binned_backward_workspace_bytes(a, dtype);
-  if (need == 0 || workspace == nullptr || workspace_bytes < need || ((uintptr_t)workspace & 255) != 0)
-    return hipErrorNotSupported;
-  const TileConfig cfg = pick_tile_config(a);
-  const int ty = cfg.ty, tx = cfg.tx;
-  const BinLayout lay = bin_layout(a, ty, tx);
+static BinWorkspace carve_workspace(void *workspace, const BinLayout &lay) {
   char *base = static_cast<char *>(workspace);
   BinWorkspace ws;
   ws.plan = reinterpret_cast<BinPlan *>(base + lay.plan);
@@ -758,28 +879,82 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
   ws.item_bin = reinterpret_cast<int *>(base + lay.item_bin);
   ws.entries = reinterpret_cast<uint32_t *>(base + lay.entries);
   ws.recs = reinterpret_cast<float4 *>(base + lay.recs);
-  const int mb = max_bins_per_bm(a.S, a.L, ty, tx);
+  return ws;
+}
 
+// plan, count, scan, fill.  `a` supplies dimensions, shapes, locations and the per-point gradient
+// buffers that receive zeros for points the operator skips.
+static hipError_t run_binning(const BwdArgs &a, const BinWorkspace &ws, int ty, int tx, hipStream_t stream) {
+  const int mb = max_bins_per_bm(a.S, a.L, ty, tx);
+  hipLaunchKernelGGL(plan_and_clear_kernel, dim3(64), dim3(256), 0, stream, ws, a.shapes, a.shape_stride, a.level_start,
+                     a.L, a.S, (a.dist != nullptr || a.C == 0) ? a.D : 0, a.B, a.M, ty, tx, a.chunk_hint > 0 ? a.chunk_hint : 1024, mb);
+  const int q_blocks = (a.Q + kBinQueries - 1) / kBinQueries;
+  const long long blocks = (long long)a.B * a.M * q_blocks;
+  if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
+  const int hist_cap = mb < kHistCap ? mb : kHistCap;
+  hipLaunchKernelGGL(bin_points_kernel<0>, dim3((unsigned)blocks), dim3(256), (size_t)hist_cap * 4, stream, ws,
+                     (const float *)a.loc, a.loc_stride, (const float *)a.attn, (float *)a.grad_loc, a.grad_loc_stride,
+                     (float *)a.grad_attn, (float *)a.grad_score_out, a.B, a.M, a.L, a.Q, a.P, q_blocks, hist_cap, a.diag);
+  hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(1024), 0, stream, ws);
+  hipLaunchKernelGGL(bin_points_kernel<1>, dim3((unsigned)blocks), dim3(256), (size_t)hist_cap * 8, stream, ws,
+                     (const float *)a.loc, a.loc_stride, (const float *)a.attn, (float *)a.grad_loc, a.grad_loc_stride,
+                     (float *)a.grad_attn, (float *)a.grad_score_out, a.B, a.M, a.L, a.Q, a.P, q_blocks, hist_cap, a.diag);
+  return hipGetLastError();
+}
+
+// Binned backward of both stages (a.dist given) or of stage 2 alone (a.dist == nullptr, a.score_in /
+// a.grad_score_out given).  Returns hipErrorNotSupported when the binned path does not apply and the
+// caller should use launch_backward instead.
+hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, size_t workspace_bytes,
+                                  hipStream_t stream) {
+  const int kind = bwd_kind(a);
+  if (dtype == DFA3D_F64) return hipErrorNotSupported;
+  if (kind == 0 && (a.loc_stride != 3 || a.grad_loc_stride != 3 || a.shape_stride != 3)) return hipErrorNotSupported;
+  const size_t need = workspace_bytes_for(a, kind, dtype);
+  if (need == 0 || workspace == nullptr || workspace_bytes < need || ((uintptr_t)workspace & 255) != 0)
+    return hipErrorNotSupported;
+  const TileConfig cfg = tile_config_of(a, kind);
+  const BinWorkspace ws = carve_workspace(workspace, bin_layout(a, cfg.ty, cfg.tx));
   if (a.stage == 0 || a.stage == 1) {
-    hipLaunchKernelGGL(plan_and_clear_kernel, dim3(64), dim3(256), 0, stream, ws, a.shapes, a.level_start, a.L, a.S,
-                       a.D, a.B, a.M, ty, tx, a.chunk_hint > 0 ? a.chunk_hint : 1024, mb);
-    const int q_blocks = (a.Q + kBinQueries - 1) / kBinQueries;
-    const long long blocks = (long long)a.B * a.M * q_blocks;
-    if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
-    const int hist_cap = mb < kHistCap ? mb : kHistCap;
-    hipLaunchKernelGGL(bin_points_kernel<0>, dim3((unsigned)blocks), dim3(256), (size_t)hist_cap * 4, stream, ws,
-                       (const float *)a.loc, (const float *)a.attn, (float *)a.grad_loc, (float *)a.grad_attn, a.B, a.M,
-                       a.L, a.Q, a.P, q_blocks, hist_cap, a.diag);
-    hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(1024), 0, stream, ws);
-    hipLaunchKernelGGL(bin_points_kernel<1>, dim3((unsigned)blocks), dim3(256), (size_t)hist_cap * 8, stream, ws,
-                       (const float *)a.loc, (const float *)a.attn, (float *)a.grad_loc, (float *)a.grad_attn, a.B, a.M,
-                       a.L, a.Q, a.P, q_blocks, hist_cap, a.diag);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, stream)) return e;
   }
   if (a.stage == 1) return hipSuccess;
   if (dtype == DFA3D_F32) return launch_tile_typed<float>(a, ws, cfg, stream);
   return launch_tile_typed<__hip_bfloat16>(a, ws, cfg, stream);
+}
+
+// Binned backward of stage 1 alone.
+size_t binned_depth_score_backward_workspace_bytes(const DepthScoreBwdArgs &d, int dtype, int tile_hint) {
+  BwdArgs a{};
+  a.B = d.B; a.S = d.S; a.M = d.M; a.C = 0; a.D = d.D; a.L = d.L; a.Q = d.Q; a.P = d.P; a.tile_hint = tile_hint;
+  return workspace_bytes_for(a, 2, dtype);
+}
+
+hipError_t launch_depth_score_backward_binned(const DepthScoreBwdArgs &d, int dtype, void *workspace,
+                                              size_t workspace_bytes, int tile_hint, int chunk_hint, hipStream_t stream) {
+  if (dtype == DFA3D_F64) return hipErrorNotSupported;
+  BwdArgs a{};
+  a.B = d.B; a.S = d.S; a.M = d.M; a.C = 0; a.D = d.D; a.L = d.L; a.Q = d.Q; a.P = d.P;
+  a.shapes = d.shapes3; a.shape_stride = 3; a.level_start = d.level_start; a.loc = d.loc3; a.loc_stride = 3;
+  a.attn = nullptr; a.grad_loc = d.grad_loc3; a.grad_loc_stride = 3; a.grad_attn = nullptr; a.grad_score_out = nullptr;
+  a.tile_hint = tile_hint; a.chunk_hint = chunk_hint;
+  const size_t need = workspace_bytes_for(a, 2, dtype);
+  if (need == 0 || workspace == nullptr || workspace_bytes < need || ((uintptr_t)workspace & 255) != 0)
+    return hipErrorNotSupported;
+  const TileConfig cfg = tile_config_of(a, 2);
+  const BinWorkspace ws = carve_workspace(workspace, bin_layout(a, cfg.ty, cfg.tx));
+  if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, stream)) return e;
+  const int grid = tile_grid(cfg.lds, cfg.block);
+  if (dtype == DFA3D_F32) {
+    hipLaunchKernelGGL(tile_depth_backward_kernel<float>, dim3(grid), dim3(cfg.block), cfg.lds, stream, ws,
+                       (const float *)d.dist, (const float *)d.grad_score, (float *)d.grad_dist, (float *)d.grad_loc3,
+                       d.B, d.S, d.M, d.D, d.L, d.Q, d.P);
+  } else {
+    hipLaunchKernelGGL(tile_depth_backward_kernel<__hip_bfloat16>, dim3(grid), dim3(cfg.block), cfg.lds, stream, ws,
+                       (const __hip_bfloat16 *)d.dist, (const __hip_bfloat16 *)d.grad_score, (float *)d.grad_dist,
+                       (float *)d.grad_loc3, d.B, d.S, d.M, d.D, d.L, d.Q, d.P);
+  }
+  return hipGetLastError();
 }
 
 }  // namespace dfa3d

@@ -206,10 +206,10 @@ __device__ __forceinline__ void load_level_table(LevelTable &tab, const int64_t 
   if ((int)threadIdx.x < L) {
     const int l = threadIdx.x;
     const int64_t H = shapes[l * shape_stride], W = shapes[l * shape_stride + 1];
-    const int64_t Dd = shape_stride > 2 ? shapes[l * shape_stride + 2] : 1;
+    const int64_t Dd = (shape_stride > 2 && D > 0) ? shapes[l * shape_stride + 2] : 1;   // D <= 0: depth extent unused
     const int64_t st = level_start[l];
     const bool ok = H > 0 && W > 0 && st >= 0 && H <= S && W <= S && st + H * W <= (int64_t)S &&
-                    Dd > 0 && (shape_stride <= 2 || Dd <= D);
+                    Dd > 0 && (D <= 0 || Dd <= D);
     tab.H[l] = ok ? (int)H : 0;
     tab.W[l] = ok ? (int)W : 0;
     tab.Dd[l] = ok ? (int)Dd : 0;
@@ -302,10 +302,32 @@ template <> struct BufPair<double> {
     x = __hiloint2double((int)t.y, (int)t.x); y = __hiloint2double((int)t.w, (int)t.z);
   }
 };
-template <> struct BufPair<__hip_bfloat16> {      // a 4-byte load may not sit on a 2-byte boundary: two loads
+template <> struct BufPair<__hip_bfloat16> {
+  // two 2-byte loads; corner_scores uses ld_aligned4 instead when rows are 8-byte aligned
   static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, float &x, float &y) {
     x = BufElem<__hip_bfloat16>::ld(r, off);
     y = BufElem<__hip_bfloat16>::ld(r, off == kNoRow ? kNoRow : off + 2);
+  }
+  // Rows that start on 8-byte boundaries (D % 4 == 0): one 8-byte load of the aligned group of four
+  // bins holds the pair unless it starts at the group's last bin (then one extra 2-byte load).
+  static __device__ __forceinline__ void ld_aligned4(rsrc_t r, uint32_t off, float &x, float &y) {
+    const bool none = off == kNoRow;
+    const uint32_t idx = (off >> 1) & 3;
+    const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, none ? kNoRow : (off & ~7u), 0, 0);
+    const uint32_t extra = __builtin_amdgcn_raw_buffer_load_b16(r, (none || idx != 3) ? kNoRow : off + 2, 0, 0);
+    const unsigned long long v = (((unsigned long long)t.y << 32) | t.x) >> (16 * idx);
+    x = bf16_bits_to_float((uint32_t)v & 0xFFFFu);
+    y = bf16_bits_to_float(idx == 3 ? (extra & 0xFFFFu) : ((uint32_t)(v >> 16) & 0xFFFFu));
+  }
+};
+
+template <typename T> struct PairLoader {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, int, T &x, T &y) { BufPair<T>::ld(r, off, x, y); }
+};
+template <> struct PairLoader<__hip_bfloat16> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, int D, float &x, float &y) {
+    if ((D & 3) == 0) BufPair<__hip_bfloat16>::ld_aligned4(r, off, x, y);
+    else BufPair<__hip_bfloat16>::ld(r, off, x, y);
   }
 };
 
@@ -324,7 +346,7 @@ __device__ __forceinline__ void corner_scores(rsrc_t dist_r, const int (&key)[4]
     for (int k = 0; k < 4; ++k) {
       const uint32_t row = (uint32_t)(((key[k] * M + m) * D + db) * (int)sizeof(T));
       A x, y;
-      BufPair<T>::ld(dist_r, (key[k] >= 0 && tap.inside) ? row : kNoRow, x, y);
+      PairLoader<T>::ld(dist_r, (key[k] >= 0 && tap.inside) ? row : kNoRow, D, x, y);
       lo[k] = lo_x ? x : lo_y ? y : (A)0;
       hi[k] = hi_x ? x : hi_y ? y : (A)0;
     }

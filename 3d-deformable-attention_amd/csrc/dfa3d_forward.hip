@@ -60,7 +60,7 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
   __shared__ LevelTable tab;
   __shared__ Task<A> s_tasks[kWavesPerBlock][kWave * 4];
 
-  load_level_table(tab, shapes, shape_stride, level_start, L, S, FUSED ? D : 1);
+  load_level_table(tab, shapes, shape_stride, level_start, L, S, FUSED ? D : 0);
 
   const WaveShape ws = wave_shape(L, P);
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;

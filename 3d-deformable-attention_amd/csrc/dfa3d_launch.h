@@ -82,9 +82,13 @@ hipError_t launch_forward(const FwdArgs &a, int dtype, hipStream_t stream);
 hipError_t launch_depth_score(const DepthScoreArgs &a, int dtype, hipStream_t stream);
 hipError_t launch_backward(const BwdArgs &a, int dtype, hipStream_t stream);
 hipError_t launch_depth_score_backward(const DepthScoreBwdArgs &a, int dtype, hipStream_t stream);
-// binned (LDS-privatised) fused backward; hipErrorNotSupported = use launch_backward instead
-size_t binned_backward_workspace_bytes(const BwdArgs &a, int dtype);
+// Binned (LDS-accumulating) backward kernels; hipErrorNotSupported = use the direct launcher instead.
+// kind 0: both stages, 1: stage 2 alone, 2: stage 1 alone.
+size_t binned_backward_workspace_bytes(const BwdArgs &a, int kind, int dtype);
 hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, size_t workspace_bytes,
                                   hipStream_t stream);
+size_t binned_depth_score_backward_workspace_bytes(const DepthScoreBwdArgs &d, int dtype, int tile_hint);
+hipError_t launch_depth_score_backward_binned(const DepthScoreBwdArgs &d, int dtype, void *workspace,
+                                              size_t workspace_bytes, int tile_hint, int chunk_hint, hipStream_t stream);
 
 }  // namespace dfa3d

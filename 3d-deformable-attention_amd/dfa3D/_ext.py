@@ -123,11 +123,14 @@ def ms_depth_score_sample_backward(value, value_spatial_shapes, value_level_star
     _step(B, im2col_step)
     if grad_output.numel() == 0:
         return
+    code = _lib.dtype_code(value)
+    ws_bytes = _lib.lib().dfa3d_ms_depth_score_sample_backward_workspace_bytes(B, S, M, D, L, Q, P, code)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
     with torch.cuda.device(dev):
         rc = _lib.lib().dfa3d_ms_depth_score_sample_backward(
             _lib.ptr(value), _lib.ptr(value_spatial_shapes), _lib.ptr(value_level_start_index),
             _lib.ptr(sampling_locations), _lib.ptr(grad_output), _lib.ptr(grad_value), _lib.ptr(grad_sampling_loc),
-            B, S, M, D, L, Q, P, _lib.dtype_code(value), _lib.stream_of(value))
+            _lib.ptr(workspace), ws_bytes, B, S, M, D, L, Q, P, code, _lib.stream_of(value))
     _lib.check(rc, "dfa3d_ms_depth_score_sample_backward")
 
 
@@ -203,12 +206,15 @@ def wms_deform_attn_backward(value, value_spatial_shapes, value_level_start_inde
     _step(B, im2col_step)
     if grad_output.numel() == 0:
         return
+    code = _lib.dtype_code(value)
+    ws_bytes = _lib.lib().dfa3d_wms_deform_attn_backward_workspace_bytes(B, S, M, C, L, Q, P, code)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
     with torch.cuda.device(dev):
         rc = _lib.lib().dfa3d_wms_deform_attn_backward(
             _lib.ptr(value), _lib.ptr(value_spatial_shapes), sw, _lib.ptr(value_level_start_index),
             _lib.ptr(sampling_locations), lw, _lib.ptr(attention_weights), _lib.ptr(depth_scores),
             _lib.ptr(grad_output), _lib.ptr(grad_value), _lib.ptr(grad_sampling_loc), gw, _lib.ptr(grad_attn_weight),
-            _lib.ptr(grad_depth_score), B, S, M, C, L, Q, P, _lib.dtype_code(value), _lib.stream_of(value))
+            _lib.ptr(grad_depth_score), _lib.ptr(workspace), ws_bytes, B, S, M, C, L, Q, P, code, _lib.stream_of(value))
     _lib.check(rc, "dfa3d_wms_deform_attn_backward")
 
 

@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdfa3d_hip.so")
 
 DFA3D_F32, DFA3D_F64, DFA3D_BF16 = 0, 1, 2
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _P, _I = ctypes.c_void_p, ctypes.c_int
 _DIMS7 = [_I] * 7      # B S M (C|D) L Q P
@@ -21,9 +21,10 @@ _DIMS8 = [_I] * 8      # B S M C D L Q P
 # name -> argument types; every entry point returns int
 SIGNATURES = {
     "dfa3d_ms_depth_score_sample_forward": [_P] * 5 + _DIMS7 + [_I, _P],
-    "dfa3d_ms_depth_score_sample_backward": [_P] * 7 + _DIMS7 + [_I, _P],
+    "dfa3d_ms_depth_score_sample_backward": [_P] * 8 + [ctypes.c_size_t] + _DIMS7 + [_I, _P],
     "dfa3d_wms_deform_attn_forward": [_P, _P, _I, _P, _P, _I, _P, _P, _P] + _DIMS7 + [_I, _P],
-    "dfa3d_wms_deform_attn_backward": [_P, _P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P] + _DIMS7 + [_I, _P],
+    "dfa3d_wms_deform_attn_backward": [_P, _P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _P, ctypes.c_size_t]
+    + _DIMS7 + [_I, _P],
     "dfa3d_fused_forward": [_P] * 8 + _DIMS8 + [_I, _P],
     "dfa3d_fused_backward": [_P] * 13 + [ctypes.c_size_t] + _DIMS8 + [_I, _P],
     "dfa3d_set_tunable": [ctypes.c_char_p, _I],
@@ -47,8 +48,12 @@ def lib():
             fn = getattr(handle, name)
             fn.argtypes = argtypes
             fn.restype = ctypes.c_int
-        handle.dfa3d_fused_backward_workspace_bytes.argtypes = _DIMS8 + [_I]
-        handle.dfa3d_fused_backward_workspace_bytes.restype = ctypes.c_size_t
+        for name, dims in (("dfa3d_fused_backward_workspace_bytes", _DIMS8),
+                           ("dfa3d_wms_deform_attn_backward_workspace_bytes", _DIMS7),
+                           ("dfa3d_ms_depth_score_sample_backward_workspace_bytes", _DIMS7)):
+            fn = getattr(handle, name)
+            fn.argtypes = dims + [_I]
+            fn.restype = ctypes.c_size_t
         handle.dfa3d_last_error.argtypes = []
         handle.dfa3d_last_error.restype = ctypes.c_char_p
         if handle.dfa3d_abi_version() != ABI_VERSION:

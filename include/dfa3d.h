@@ -57,14 +57,19 @@ int dfa3d_ms_depth_score_sample_forward(
     int B, int S, int M, int D, int L, int Q, int P, int dtype, void *stream);
 
 /* Stage 1 backward.  `grad_dist` is ACCUMULATED into (caller zero-fills); every element of
- * `grad_loc3` is overwritten, its x and y components with 0.
+ * `grad_loc3` is overwritten, its x and y components with 0.  `workspace` as for
+ * dfa3d_fused_backward (size from dfa3d_ms_depth_score_sample_backward_workspace_bytes; NULL =
+ * every update is a device-memory atomic).
  * Replaces ms_depth_score_sample_backward
  * (pybind.cpp:60-66 -> ms_depth_score_sample_cuda.cu:137-202). */
 int dfa3d_ms_depth_score_sample_backward(
     const void *dist, const int64_t *shapes3, const int64_t *level_start, const void *loc3,
     const void *grad_score,
     void *grad_dist, void *grad_loc3,
+    void *workspace, size_t workspace_bytes,
     int B, int S, int M, int D, int L, int Q, int P, int dtype, void *stream);
+size_t dfa3d_ms_depth_score_sample_backward_workspace_bytes(int B, int S, int M, int D, int L, int Q, int P,
+                                                            int dtype);
 
 /* Stage 2 forward: depth-weighted multi-scale deformable attention.  Writes every element of
  * `out`.  Replaces wms_deform_attn_forward
@@ -75,15 +80,19 @@ int dfa3d_wms_deform_attn_forward(
     void *out,
     int B, int S, int M, int C, int L, int Q, int P, int dtype, void *stream);
 
-/* Stage 2 backward.  `grad_value` is ACCUMULATED into (caller zero-fills); `grad_loc`
- * (B,Q,M,L,P,grad_loc_stride) gets its first two components overwritten, `grad_attn` and
- * `grad_score` are overwritten.  Replaces wms_deform_attn_backward
+/* Stage 2 backward.  `grad_value` must be zero on entry and holds the gradient on return;
+ * `grad_loc` (B,Q,M,L,P,grad_loc_stride) gets its first two components overwritten, `grad_attn` and
+ * `grad_score` are overwritten.  `workspace` as for dfa3d_fused_backward (size from
+ * dfa3d_wms_deform_attn_backward_workspace_bytes; NULL = device-memory atomics).
+ * Replaces wms_deform_attn_backward
  * (pybind.cpp:48-54 -> wms_deform_attn_cuda.cu:291-370). */
 int dfa3d_wms_deform_attn_backward(
     const void *value, const int64_t *shapes, int shape_stride, const int64_t *level_start,
     const void *loc, int loc_stride, const void *attn, const void *score, const void *grad_out,
     void *grad_value, void *grad_loc, int grad_loc_stride, void *grad_attn, void *grad_score,
+    void *workspace, size_t workspace_bytes,
     int B, int S, int M, int C, int L, int Q, int P, int dtype, void *stream);
+size_t dfa3d_wms_deform_attn_backward_workspace_bytes(int B, int S, int M, int C, int L, int Q, int P, int dtype);
 
 /* Both stages in one kernel: what the reference's one-stage autograd Function does with two
  * native calls and two slice copies
@@ -98,8 +107,8 @@ int dfa3d_fused_forward(
 /* Backward of dfa3d_fused_forward (…_function.py:306-352: two native calls, six zero fills and
  * a host synchronisation in the reference).  The depth scores are recomputed from `dist`, not
  * read back.  `grad_score_in` (may be NULL) is an incoming gradient with respect to the `score`
- * output and is chained into grad_dist and the z gradient.  `grad_value` and `grad_dist` are
- * ACCUMULATED into (caller zero-fills); `grad_loc3` and `grad_attn` are overwritten.
+ * output and is chained into grad_dist and the z gradient.  `grad_value` and `grad_dist` must be
+ * zero on entry and hold the gradients on return; `grad_loc3` and `grad_attn` are overwritten.
  *
  * `workspace` (may be NULL) is caller-owned scratch device memory, 256-byte aligned, of at least
  * dfa3d_fused_backward_workspace_bytes(...) bytes, whose contents need not be preserved or

@@ -173,6 +173,49 @@ def test_fp32_workloads_match_checker(oracle, name):
     _compare(_gpu_one_stage(inp, dev), _oracle_one_stage(oracle, inp), F32_FWD, F32_BWD)
 
 
+def _gpu_two_stage(inp, dev, sliced):
+    """The reference's two-stage composition; `sliced` hands the 2-D stage (L,2) shapes and (…,2)
+    locations as the reference does, otherwise the 3-wide tensors go in as they are."""
+    _, F3, F2 = _functions()
+    value = inp["value"].to(dev).requires_grad_()
+    dist = inp["value_dpt_dist"].to(dev).requires_grad_()
+    loc3 = inp["sampling_locations"].to(dev).requires_grad_()
+    attn = inp["attention_weights"].to(dev).requires_grad_()
+    shapes3, lsi = inp["spatial_shapes"].to(dev), inp["level_start_index"].to(dev)
+    score = F3.apply(dist, shapes3, lsi, loc3, 64)
+    if sliced:
+        out = F2.apply(value, shapes3[:, :2].contiguous(), lsi, loc3[..., :2].contiguous(), attn, score, 64)
+    else:
+        out = F2.apply(value, shapes3, lsi, loc3, attn, score, 64)
+    gv, gd, gl, ga = torch.autograd.grad(out, [value, dist, loc3, attn], inp["grad_output"].to(dev))
+    torch.cuda.synchronize()
+    return out.detach().cpu(), score.detach().cpu(), gv.cpu(), gd.cpu(), gl.cpu(), ga.cpu()
+
+
+@pytest.mark.parametrize("binned", [1, 0], ids=["tiles", "atomics"])
+@pytest.mark.parametrize("sliced", [True, False], ids=["sliced", "wide"])
+def test_fp32_two_stage_workloads_match_checker(oracle, binned, sliced):
+    """Both backward implementations of the two separate stages (LDS tiles with a workspace, and
+    device-memory atomics), with 2-wide and 3-wide shape / location operands."""
+    from dfa3D import _lib
+    from dfa3D.workloads import WORKLOADS, make_inputs
+    dev = _dev()
+    _lib.set_tunable("binned", binned)
+    try:
+        for name in ("unit", "small"):
+            inp = make_inputs(WORKLOADS[name])
+            _compare(_gpu_two_stage(inp, dev, sliced), _oracle_one_stage(oracle, inp), F32_FWD, F32_BWD)
+    finally:
+        _lib.set_tunable("binned", 1)
+
+
+def test_fp32_base_shape_two_stage_matches_checker(oracle):
+    from dfa3D.workloads import WORKLOADS, make_inputs
+    dev = _dev()
+    inp = make_inputs(WORKLOADS["base"])
+    _compare(_gpu_two_stage(inp, dev, sliced=False), _oracle_one_stage(oracle, inp), F32_FWD, F32_BWD)
+
+
 def test_fp32_base_shape_matches_checker(oracle):
     """BEVFormer-base shape at full size (15.36 M sampling points)."""
     from dfa3D.workloads import WORKLOADS, make_inputs

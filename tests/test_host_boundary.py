@@ -53,7 +53,7 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     assert rc == -1 and b"NULL" in L.dfa3d_last_error()
     rc = L.dfa3d_wms_deform_attn_forward(one, one, 4, one, one, 2, one, one, one, 1, 10, 8, 32, 2, 5, 4, 0, null)
     assert rc == -1 and b"stride" in L.dfa3d_last_error()
-    rc = L.dfa3d_ms_depth_score_sample_backward(one, one, one, one, one, null, one, 1, 10, 8, 16, 2, 5, 4, 0, null)
+    rc = L.dfa3d_ms_depth_score_sample_backward(one, one, one, one, one, null, one, null, 0, 1, 10, 8, 16, 2, 5, 4, 0, null)
     assert rc == -1 and b"grad_dist" in L.dfa3d_last_error()
     assert L.dfa3d_set_tunable(b"iters", 0) == -1
     assert L.dfa3d_set_tunable(b"nope", 1) == -1
