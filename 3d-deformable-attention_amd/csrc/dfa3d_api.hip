@@ -92,7 +92,7 @@ int dfa3d_stream_copy(void *dst, const void *src, size_t bytes, void *stream) {
 }
 
 const char *dfa3d_last_error(void) { return g_err; }
-int dfa3d_abi_version(void) { return 3; }
+int dfa3d_abi_version(void) { return 4; }
 
 int dfa3d_set_tunable(const char *name, int value) {
   if (name == nullptr) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: name is NULL");
@@ -254,16 +254,18 @@ int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int
 }
 
 int dfa3d_fused_forward(const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
-                        const void *loc3, const void *attn, void *out, void *score, int B, int S, int M, int C, int D,
-                        int L, int Q, int P, int dtype, void *stream) {
+                        const void *loc3, const void *attn, void *out, void *score, void *weight_update, int B, int S,
+                        int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype, void *stream) {
   const char *fn = "dfa3d_fused_forward";
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  if (dist_heads != M && dist_heads != 1) return fail(DFA3D_EINVAL, "%s: dist_heads must be M or 1", fn);
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
   REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, out);
   dfa3d::FwdArgs a{};
   a.value = value; a.dist = dist; a.shapes = shapes3; a.shape_stride = 3; a.level_start = level_start;
   a.loc = loc3; a.loc_stride = 3; a.attn = attn; a.score_in = nullptr; a.out = out; a.score_out = score;
+  a.weight_update = weight_update; a.dist_heads = dist_heads;
   a.B = B; a.S = S; a.M = M; a.C = C; a.D = D; a.L = L; a.Q = Q; a.P = P;
   a.iters = tune_iters(); a.vec_hint = tune_vec();
   return hip_result(dfa3d::launch_forward(a, dtype, (hipStream_t)stream), fn);
@@ -271,14 +273,15 @@ int dfa3d_fused_forward(const void *value, const void *dist, const int64_t *shap
 
 static dfa3d::BwdArgs fused_bwd_args(const void *value, const void *dist, const int64_t *shapes3,
                                      const int64_t *level_start, const void *loc3, const void *attn,
-                                     const void *grad_out, const void *grad_score_in, void *grad_value,
-                                     void *grad_dist, void *grad_loc3, void *grad_attn, int B, int S, int M, int C,
-                                     int D, int L, int Q, int P) {
+                                     const void *grad_out, const void *grad_score_in, const void *grad_weight_update,
+                                     void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn, int B, int S,
+                                     int M, int C, int D, int L, int Q, int P, int dist_heads) {
   dfa3d::BwdArgs a{};
   a.value = value; a.dist = dist; a.shapes = shapes3; a.shape_stride = 3; a.level_start = level_start;
   a.loc = loc3; a.loc_stride = 3; a.attn = attn; a.score_in = nullptr; a.grad_out = grad_out;
   a.grad_score_in = grad_score_in; a.grad_value = grad_value; a.grad_dist = grad_dist; a.grad_loc = grad_loc3;
   a.grad_loc_stride = 3; a.grad_attn = grad_attn; a.grad_score_out = nullptr;
+  a.grad_weight_update = grad_weight_update; a.dist_heads = dist_heads;
   a.B = B; a.S = S; a.M = M; a.C = C; a.D = D; a.L = L; a.Q = Q; a.P = P;
   a.iters = tune_iters(); a.vec_hint = tune_vec(); a.diag = g_diag.load(std::memory_order_relaxed);
   a.tile_hint = g_tile.load(std::memory_order_relaxed); a.block_hint = g_block.load(std::memory_order_relaxed);
@@ -293,23 +296,25 @@ size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, i
   if (check_dims("dfa3d_fused_backward_workspace_bytes", B, S, M, D, L, Q, P, dtype)) return 0;
   if (!g_binned.load(std::memory_order_relaxed)) return 0;
   const dfa3d::BwdArgs a = fused_bwd_args(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
-                                          nullptr, nullptr, nullptr, nullptr, B, S, M, C, D, L, Q, P);
+                                          nullptr, nullptr, nullptr, nullptr, nullptr, B, S, M, C, D, L, Q, P, M);
   return dfa3d::binned_backward_workspace_bytes(a, 0, dtype);
 }
 
 int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
                          const void *loc3, const void *attn, const void *grad_out, const void *grad_score_in,
-                         void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn,
-                         void *workspace, size_t workspace_bytes, int B, int S, int M,
-                         int C, int D, int L, int Q, int P, int dtype, void *stream) {
+                         const void *grad_weight_update, void *grad_value, void *grad_dist, void *grad_loc3,
+                         void *grad_attn, void *workspace, size_t workspace_bytes, int B, int S, int M,
+                         int C, int D, int L, int Q, int P, int dist_heads, int dtype, void *stream) {
   const char *fn = "dfa3d_fused_backward";
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  if (dist_heads != M && dist_heads != 1) return fail(DFA3D_EINVAL, "%s: dist_heads must be M or 1", fn);
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
   REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
   REQUIRE_PTR(fn, grad_dist); REQUIRE_PTR(fn, grad_loc3); REQUIRE_PTR(fn, grad_attn);
   const dfa3d::BwdArgs a = fused_bwd_args(value, dist, shapes3, level_start, loc3, attn, grad_out, grad_score_in,
-                                          grad_value, grad_dist, grad_loc3, grad_attn, B, S, M, C, D, L, Q, P);
+                                          grad_weight_update, grad_value, grad_dist, grad_loc3, grad_attn, B, S, M, C,
+                                          D, L, Q, P, dist_heads);
   if (workspace != nullptr && g_binned.load(std::memory_order_relaxed)) {
     const hipError_t e = dfa3d::launch_backward_binned(a, dtype, workspace, workspace_bytes, (hipStream_t)stream);
     if (e != hipErrorNotSupported) return hip_result(e, fn);

@@ -124,6 +124,7 @@ __global__ __launch_bounds__(kBlock) void bwd_attention_kernel(
     const A *__restrict__ attn, const T *__restrict__ score_in, const T *__restrict__ grad_out,
     const T *__restrict__ grad_score_in, A *__restrict__ grad_value, A *__restrict__ grad_dist,
     A *__restrict__ grad_loc, int gl_stride, A *__restrict__ grad_attn, A *__restrict__ grad_score_out,
+    const A *__restrict__ grad_wu, int Md,
     int B, int S, int M, int C, int D, int L, int Q, int P, int iters, int q_blocks, int diag) {
   __shared__ LevelTable tab;
   __shared__ Task<A> s_tasks[kWavesPerBlock][kWave * 4];
@@ -142,12 +143,13 @@ __global__ __launch_bounds__(kBlock) void bwd_attention_kernel(
   A *dots = s_dots[wave];
 
   A *gvalue_b = grad_value + (size_t)b * S * M * C;
-  A *gdist_b = FUSED ? grad_dist + (size_t)b * S * M * D : nullptr;
+  A *gdist_b = FUSED ? grad_dist + (size_t)b * S * Md * D : nullptr;
+  const int md = Md == 1 ? 0 : m;
   const rsrc_t value_r = make_rsrc(value + (size_t)b * S * M * C, (size_t)S * M * C * sizeof(T));
   const rsrc_t gvalue_r = make_rsrc(gvalue_b, (diag & 1) ? 0 : (size_t)S * M * C * sizeof(A));
-  const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * M * D : nullptr,
-                                  FUSED ? (size_t)S * M * D * sizeof(T) : 0);
-  const rsrc_t gdist_r = make_rsrc(gdist_b, (FUSED && !(diag & 2)) ? (size_t)S * M * D * sizeof(A) : 0);
+  const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * Md * D : nullptr,
+                                  FUSED ? (size_t)S * Md * D * sizeof(T) : 0);
+  const rsrc_t gdist_r = make_rsrc(gdist_b, (FUSED && !(diag & 2)) ? (size_t)S * Md * D * sizeof(A) : 0);
   const int q_per_iter = kWavesPerBlock * ws.upw;
 
   for (int it = 0; it < iters; ++it) {
@@ -180,7 +182,7 @@ __global__ __launch_bounds__(kBlock) void bwd_attention_kernel(
         g = locate_2d<A>(pl[0], pl[1], tab.H[l], tab.W[l], tab.start[l]);
         if (FUSED) {
           tap = locate_depth<A>(pl[2], tab.Dd[l]);
-          corner_scores<T, A>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
+          corner_scores<T, A>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
         } else {
           const T *si = score_in + gp * 4;
 #pragma unroll
@@ -252,11 +254,17 @@ __global__ __launch_bounds__(kBlock) void bwd_attention_kernel(
 #pragma unroll
             for (int k = 0; k < 4; ++k) gs[k] += Elem<T>::ld(gi + k);
           }
+          if (grad_wu != nullptr) {       // weight_update = sum over points of attn * mean corner score
+            const A gw = grad_wu[gp / ws.LP] * (A)0.25;
+            grad_attn[gp] = ga + gw * (sc[0] + sc[1] + sc[2] + sc[3]);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) gs[k] += gw * a;
+          }
           A gz = 0;
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
             const bool on = g.key[k] >= 0 && gs[k] != 0;
-            const uint32_t row = (uint32_t)(((g.key[k] * M + m) * D + tap.d0) * (int)sizeof(A));
+            const uint32_t row = (uint32_t)(((g.key[k] * Md + md) * D + tap.d0) * (int)sizeof(A));
             scatter_add(gdist_r, gdist_b, (on && tap.lo_ok) ? row : kNoRow, tap.hd * gs[k]);
             scatter_add(gdist_r, gdist_b, (on && tap.hi_ok) ? row + (uint32_t)sizeof(A) : kNoRow, tap.ld * gs[k]);
             gz += (g.key[k] >= 0 && tap.inside) ? gs[k] * (hi[k] - lo[k]) : (A)0;
@@ -333,15 +341,16 @@ static hipError_t launch_bwd_cfg(const BwdArgs &a, hipStream_t stream) {
                        (const T *)a.value, (const T *)a.dist, a.shapes, a.shape_stride, a.level_start,
                        (const A *)a.loc, a.loc_stride, (const A *)a.attn, (const T *)nullptr,
                        (const T *)a.grad_out, (const T *)a.grad_score_in, (A *)a.grad_value, (A *)a.grad_dist,
-                       (A *)a.grad_loc, a.grad_loc_stride, (A *)a.grad_attn, (A *)nullptr, a.B, a.S, a.M, a.C, a.D,
+                       (A *)a.grad_loc, a.grad_loc_stride, (A *)a.grad_attn, (A *)nullptr,
+                       (const A *)a.grad_weight_update, a.dist_heads == 1 ? 1 : a.M, a.B, a.S, a.M, a.C, a.D,
                        a.L, a.Q, a.P, iters, q_blocks, a.diag);
   } else {
     hipLaunchKernelGGL((bwd_attention_kernel<T, A, VEC, LPR, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,
                        (const T *)a.value, (const T *)nullptr, a.shapes, a.shape_stride, a.level_start,
                        (const A *)a.loc, a.loc_stride, (const A *)a.attn, (const T *)a.score_in,
                        (const T *)a.grad_out, (const T *)nullptr, (A *)a.grad_value, (A *)nullptr, (A *)a.grad_loc,
-                       a.grad_loc_stride, (A *)a.grad_attn, (A *)a.grad_score_out, a.B, a.S, a.M, a.C, a.D, a.L, a.Q,
-                       a.P, iters, q_blocks, a.diag);
+                       a.grad_loc_stride, (A *)a.grad_attn, (A *)a.grad_score_out, (const A *)nullptr, a.M, a.B, a.S,
+                       a.M, a.C, a.D, a.L, a.Q, a.P, iters, q_blocks, a.diag);
   }
   return hipGetLastError();
 }

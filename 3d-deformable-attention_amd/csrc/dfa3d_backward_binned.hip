@@ -310,7 +310,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
     BinWorkspace ws, const T *__restrict__ value, const T *__restrict__ dist, const T *__restrict__ score_in,
     const T *__restrict__ grad_out, const T *__restrict__ grad_score_in,
     float *__restrict__ grad_value, float *__restrict__ grad_dist, float *__restrict__ grad_loc, int gl_stride,
-    float *__restrict__ grad_attn, float *__restrict__ grad_score_out,
+    float *__restrict__ grad_attn, float *__restrict__ grad_score_out, const float *__restrict__ grad_wu, int Md,
     int B, int S, int M, int C, int D, int L, int Q, int P, int PP, int diag) {
   constexpr int RPI = kWave / LPR;                  // row groups per wavefront
   extern __shared__ __align__(16) float smem[];
@@ -365,7 +365,8 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
     const int y0 = (tile / p.tiles_x[l]) * TY, x0 = (tile % p.tiles_x[l]) * TX;
 
     const rsrc_t value_r = make_rsrc(value + (size_t)b * S * M * C, (size_t)S * M * C * sizeof(T));
-    const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * M * D : nullptr, FUSED ? (size_t)S * M * D * sizeof(T) : 0);
+    const int md = Md == 1 ? 0 : m;
+    const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * Md * D : nullptr, FUSED ? (size_t)S * Md * D * sizeof(T) : 0);
     const rsrc_t go_r = make_rsrc(grad_out + (size_t)b * Q * M * C, (size_t)Q * M * C * sizeof(T));
 
     for (int base = 0; base < n_item; base += PP) {               // uniform over the workgroup
@@ -391,7 +392,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         g = locate_2d<float>(rec.x, rec.y, H, W, start);
         if (FUSED) {
           tap = locate_depth<float>(rec.z, Dd);
-          corner_scores<T, float>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
+          corner_scores<T, float>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
         } else {
           const T *si = score_in + gp * 4;
 #pragma unroll
@@ -553,12 +554,17 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const float gy = (float)H * a * (g.hw * (s[3] - s[0]) + g.lw * (s[2] - s[1]));
         float *gl = grad_loc + gp * gl_stride;
         gl[0] = gx; gl[1] = gy;
-        grad_attn[gp] = ga;
         if (FUSED) {
           if (grad_score_in != nullptr) {
             const T *gi = grad_score_in + gp * 4;
 #pragma unroll
             for (int k = 0; k < 4; ++k) gs[k] += Elem<T>::ld(gi + k);
+          }
+          if (grad_wu != nullptr) {       // weight_update = sum over points of attn * mean corner score
+            const float gw = grad_wu[gp / LP] * 0.25f;
+            ga += gw * (sc[0] + sc[1] + sc[2] + sc[3]);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) gs[k] += gw * a;
           }
           float gz = 0;
 #pragma unroll
@@ -576,6 +582,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
 #pragma unroll
           for (int k = 0; k < 4; ++k) go4[k] = gs[k];
         }
+        grad_attn[gp] = ga;
       }
       __syncthreads();                                   // before the next pass reuses the scratch arrays
       TT_MARK(5);
@@ -583,13 +590,14 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
 
     // ---------------- flush the tile (and leave it zeroed for the next item) ----------------
     float *gvalue_b = grad_value + (size_t)b * S * M * C;
-    float *gdist_b = FUSED ? grad_dist + (size_t)b * S * M * D : nullptr;
+    float *gdist_b = FUSED ? grad_dist + (size_t)b * S * Md * D : nullptr;
     const rsrc_t gvalue_r = make_rsrc(gvalue_b, (size_t)S * M * C * sizeof(float));
-    const rsrc_t gdist_r = make_rsrc(gdist_b, FUSED ? (size_t)S * M * D * sizeof(float) : 0);
+    const rsrc_t gdist_r = make_rsrc(gdist_b, FUSED ? (size_t)S * Md * D * sizeof(float) : 0);
     // Rows 1..TY-1 x 1..TX-1 of the tile belong to no neighbour's halo; when this item holds all the
     // points of its bin nobody else adds to them, so they are stored instead of added atomically
     // (grad_value and grad_dist are zero on entry).
     const bool sole = chunks_here == 1;
+    const bool sole_d = sole && Md == M;                 // a distribution shared by the heads collects from all of them
     if (((C | D) & 3) == 0) {
       // four floats per lane: whole 128-byte lines leave each row group at once
       const int c4n = C >> 2, d4n = D >> 2;
@@ -620,8 +628,8 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const int ry = r / TW, rx = r - ry * TW;
         const int y = y0 + ry, x = x0 + rx;
         if (y < H && x < W && !(diag & 4)) {
-          const uint32_t off = (uint32_t)((((start + y * W + x) * M + m) * D + d) * 4);
-          if (sole && ry >= 1 && ry < TY && rx >= 1 && rx < TX) {
+          const uint32_t off = (uint32_t)((((start + y * W + x) * Md + md) * D + d) * 4);
+          if (sole_d && ry >= 1 && ry < TY && rx >= 1 && rx < TX) {
             *reinterpret_cast<float4 *>(gdist_b + (off >> 2)) = val;
           } else if (nz) {
             if (val.x != 0) scatter_add(gdist_r, gdist_b, off, val.x);
@@ -649,7 +657,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const int r = i / D, d = i - r * D;
         const int ry = r / TW, rx = r % TW;
         const int y = y0 + ry, x = x0 + rx;
-        if (y < H && x < W && !(diag & 4)) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * M + m) * D + d) * 4), val);
+        if (y < H && x < W && !(diag & 4)) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * Md + md) * D + d) * 4), val);
       }
     }
     }
@@ -846,14 +854,16 @@ static hipError_t launch_tile_cfg(const BwdArgs &a, const BinWorkspace &ws, cons
     hipLaunchKernelGGL(kern, dim3(grid), dim3(c.block), c.lds, stream, ws, (const T *)a.value, (const T *)a.dist,
                        (const T *)nullptr, (const T *)a.grad_out, (const T *)a.grad_score_in, (float *)a.grad_value,
                        (float *)a.grad_dist, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
-                       (float *)nullptr, a.B, a.S, a.M, a.C, a.D, a.L, a.Q, a.P, c.pp, a.diag);
+                       (float *)nullptr, (const float *)a.grad_weight_update, a.dist_heads == 1 ? 1 : a.M, a.B, a.S,
+                       a.M, a.C, a.D, a.L, a.Q, a.P, c.pp, a.diag);
   } else {
     auto kern = tile_backward_kernel<T, VEC, LPR, false>;
     if (hipError_t e = allow_lds(kern, c.lds)) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(c.block), c.lds, stream, ws, (const T *)a.value, (const T *)nullptr,
                        (const T *)a.score_in, (const T *)a.grad_out, (const T *)nullptr, (float *)a.grad_value,
                        (float *)nullptr, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
-                       (float *)a.grad_score_out, a.B, a.S, a.M, a.C, 0, a.L, a.Q, a.P, c.pp, a.diag);
+                       (float *)a.grad_score_out, (const float *)nullptr, a.M, a.B, a.S, a.M, a.C, 0, a.L, a.Q, a.P,
+                       c.pp, a.diag);
   }
   return hipGetLastError();
 }

@@ -56,7 +56,8 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
     const T *__restrict__ value, const T *__restrict__ dist, const int64_t *__restrict__ shapes, int shape_stride,
     const int64_t *__restrict__ level_start, const A *__restrict__ loc, int loc_stride,
     const A *__restrict__ attn, const T *__restrict__ score_in, T *__restrict__ out, T *__restrict__ score_out,
-    int B, int S, int M, int C, int D, int L, int Q, int P, int iters, int q_blocks) {
+    A *__restrict__ weight_update, int Md, int B, int S, int M, int C, int D, int L, int Q, int P, int iters,
+    int q_blocks) {
   __shared__ LevelTable tab;
   __shared__ Task<A> s_tasks[kWavesPerBlock][kWave * 4];
 
@@ -72,13 +73,15 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
   Task<A> *tasks = s_tasks[wave];
 
   const rsrc_t value_r = make_rsrc(value + (size_t)b * S * M * C, (size_t)S * M * C * sizeof(T));
-  const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * M * D : nullptr,
-                                  FUSED ? (size_t)S * M * D * sizeof(T) : 0);
+  const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * Md * D : nullptr,
+                                  FUSED ? (size_t)S * Md * D * sizeof(T) : 0);
+  const int md = Md == 1 ? 0 : m;                                    // head whose distribution this head reads
   const int q_per_iter = kWavesPerBlock * ws.upw;
 
   for (int it = 0; it < iters; ++it) {
     const int q0 = (qb * iters + it) * q_per_iter + wave * ws.upw;   // first query of this wave's group
     if (q0 >= Q) break;                                              // wave-uniform
+    A wu_unit = 0;                                                   // upw == 1: the unit's sum over its chunks
     for (int pass = 0; pass < passes; ++pass) {
       const int chan = (pass * LPR + cl) * VEC;
       const bool chan_ok = chan < C;
@@ -94,6 +97,7 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
         const int q = q0 + ul;
         const bool live = ul < ws.upw && q < Q;
         Task<A> t4[4];
+        A wu = 0;
 #pragma unroll
         for (int k = 0; k < 4; ++k) { t4[k].off = kNoRow; t4[k].w = 0; }
         if (live) {
@@ -107,12 +111,13 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
           if (FUSED) {
             A lo[4], hi[4];
             const DepthTap<A> tap = locate_depth<A>(pl[2], tab.Dd[l]);
-            corner_scores<T, A>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
+            corner_scores<T, A>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
             if (score_out != nullptr && pass == 0) {
               T *so = score_out + gp * 4;
 #pragma unroll
               for (int k = 0; k < 4; ++k) Elem<T>::st(so + k, sc[k]);
             }
+            wu = a * ((sc[0] + sc[1] + sc[2] + sc[3]) * (A)0.25);
           } else {
             const T *si = score_in + gp * 4;
 #pragma unroll
@@ -124,6 +129,20 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
               t4[k].off = (uint32_t)((g.key[k] * M + m) * C * (int)sizeof(T));
               t4[k].w = g.bil(k) * sc[k] * a;
             }
+          }
+        }
+        if (FUSED && weight_update != nullptr && pass == 0) {      // wave-uniform
+          // sum over the lanes of each unit: lane i gathers lanes [i, i + 2^k) of its own unit
+          const int seg = ws.upw == 1 ? kWave : ws.LP, pos = ws.upw == 1 ? lane : lp;
+          for (int off = 1; off < seg; off <<= 1) {
+            const A up = __shfl_down(wu, off, kWave);
+            if (pos + off < seg) wu += up;
+          }
+          if (ws.upw == 1) {
+            wu_unit += wu;                                         // lane 0 holds the chunk's sum
+            if (chunk == ws.chunks - 1 && lane == 0) weight_update[((size_t)b * Q + q0) * M + m] = wu_unit;
+          } else if (live && lp == 0) {
+            weight_update[((size_t)b * Q + q) * M + m] = wu;
           }
         }
         wave_lds_handover();     // previous phase B has consumed the task list
@@ -214,12 +233,13 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
     hipLaunchKernelGGL((fwd_attention_kernel<T, A, VEC, LPR, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,
                        (const T *)a.value, (const T *)a.dist, a.shapes, a.shape_stride, a.level_start,
                        (const A *)a.loc, a.loc_stride, (const A *)a.attn, (const T *)nullptr, (T *)a.out,
-                       (T *)a.score_out, a.B, a.S, a.M, a.C, a.D, a.L, a.Q, a.P, iters, q_blocks);
+                       (T *)a.score_out, (A *)a.weight_update, a.dist_heads == 1 ? 1 : a.M, a.B, a.S, a.M, a.C, a.D,
+                       a.L, a.Q, a.P, iters, q_blocks);
   } else {
     hipLaunchKernelGGL((fwd_attention_kernel<T, A, VEC, LPR, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,
                        (const T *)a.value, (const T *)nullptr, a.shapes, a.shape_stride, a.level_start,
                        (const A *)a.loc, a.loc_stride, (const A *)a.attn, (const T *)a.score_in, (T *)a.out,
-                       (T *)nullptr, a.B, a.S, a.M, a.C, a.D, a.L, a.Q, a.P, iters, q_blocks);
+                       (T *)nullptr, (A *)nullptr, a.M, a.B, a.S, a.M, a.C, a.D, a.L, a.Q, a.P, iters, q_blocks);
   }
   return hipGetLastError();
 }

@@ -42,6 +42,8 @@ struct FwdArgs {
   const void *loc; int loc_stride;
   const void *attn, *score_in;
   void *out, *score_out;             // score_out may be nullptr
+  void *weight_update;               // (B,Q,M) sum over a unit's points of attn * mean corner score, or nullptr
+  int dist_heads;                    // heads stored in dist: M, or 1 for one distribution shared by all heads
   int B, S, M, C, D, L, Q, P;
   int iters;                         // groups of units each wavefront walks through
   int vec_hint;
@@ -61,6 +63,8 @@ struct BwdArgs {
   const void *attn, *score_in, *grad_out, *grad_score_in;
   void *grad_value, *grad_dist, *grad_loc; int grad_loc_stride;
   void *grad_attn, *grad_score_out;
+  const void *grad_weight_update;    // gradient arriving at the forward's weight_update output, or nullptr
+  int dist_heads;                    // as in FwdArgs; grad_dist has the same head count
   int B, S, M, C, D, L, Q, P;
   int iters;
   int vec_hint;

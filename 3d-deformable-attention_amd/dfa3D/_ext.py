@@ -219,9 +219,10 @@ def wms_deform_attn_backward(value, value_spatial_shapes, value_level_start_inde
 
 
 def _fused_dims(value, dist, shapes3, lsi, loc3, attn, name):
-    if value.dim() != 4 or dist.dim() != 4 or value.shape[:3] != dist.shape[:3]:
-        raise RuntimeError(f"{name}: value (bs, keys, heads, C) and value_dpt_dist (bs, keys, heads, D) must agree on "
-                           f"their first three dimensions, got {tuple(value.shape)} and {tuple(dist.shape)}")
+    if value.dim() != 4 or dist.dim() != 4 or value.shape[:2] != dist.shape[:2] or \
+            dist.shape[2] not in (1, value.shape[2]):
+        raise RuntimeError(f"{name}: value (bs, keys, heads, C) and value_dpt_dist (bs, keys, heads or 1, D) must "
+                           f"agree on bs and keys, got {tuple(value.shape)} and {tuple(dist.shape)}")
     _expect(dist, "value_dpt_dist", dtype=value.dtype)
     B, S, M, C = value.shape
     D = dist.shape[3]
@@ -234,8 +235,11 @@ def _fused_dims(value, dist, shapes3, lsi, loc3, attn, name):
 
 
 def dfa3d_fused_forward(value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
-                        attention_weights, im2col_step, need_depth_score=True):
-    """One-kernel DFA3D forward -> (output (bs, Q, heads*C), depth_score (bs, Q, heads, L, P, 4) or None)."""
+                        attention_weights, im2col_step, need_depth_score=True, need_weight_update=False):
+    """One-kernel DFA3D forward -> (output (bs, Q, heads*C), depth_score (bs, Q, heads, L, P, 4) or None), and
+    with ``need_weight_update`` a third result, weight_update (bs, Q, heads, 1) = sum over levels and points of
+    attention weight * mean corner score.  ``value_dpt_dist`` is (bs, keys, heads, D), or (bs, keys, 1, D) for one
+    distribution shared by all heads."""
     _contig(value=value, value_dpt_dist=value_dpt_dist, spatial_shapes=value_spatial_shapes,
             level_start_index=value_level_start_index, sampling_loc=sampling_locations, attn_weight=attention_weights)
     dev = _on_gpu(value=value, value_dpt_dist=value_dpt_dist, spatial_shapes=value_spatial_shapes,
@@ -246,22 +250,24 @@ def dfa3d_fused_forward(value, value_dpt_dist, value_spatial_shapes, value_level
     _step(B, im2col_step)
     out = torch.empty(B, Q, M * C, dtype=value.dtype, device=dev)
     score = torch.empty(B, Q, M, L, P, 4, dtype=value.dtype, device=dev) if need_depth_score else None
+    wu = torch.empty(B, Q, M, 1, dtype=_aux_dtype(value.dtype), device=dev) if need_weight_update else None
     if out.numel() == 0:
-        return out, score
+        return (out, score, wu) if need_weight_update else (out, score)
     with torch.cuda.device(dev):
         rc = _lib.lib().dfa3d_fused_forward(
             _lib.ptr(value), _lib.ptr(value_dpt_dist), _lib.ptr(value_spatial_shapes),
             _lib.ptr(value_level_start_index), _lib.ptr(sampling_locations), _lib.ptr(attention_weights),
-            _lib.ptr(out), _lib.ptr(score), B, S, M, C, D, L, Q, P, _lib.dtype_code(value), _lib.stream_of(value))
+            _lib.ptr(out), _lib.ptr(score), _lib.ptr(wu), B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2],
+            _lib.dtype_code(value), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_fused_forward")
-    return out, score
+    return (out, score, wu) if need_weight_update else (out, score)
 
 
 def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
                          attention_weights, grad_output, grad_depth_score, grad_value, grad_value_dpt_dist,
-                         grad_sampling_loc, grad_attn_weight, im2col_step):
-    """One-kernel DFA3D backward.  ``grad_depth_score`` (gradient arriving at the depth_score output)
-    may be None.  Accumulates into ``grad_value`` / ``grad_value_dpt_dist`` (pre-zeroed by the caller);
+                         grad_sampling_loc, grad_attn_weight, im2col_step, grad_weight_update=None):
+    """One-kernel DFA3D backward.  ``grad_depth_score`` and ``grad_weight_update`` (gradients arriving at the
+    depth_score and weight_update outputs) may be None.  Accumulates into ``grad_value`` / ``grad_value_dpt_dist`` (pre-zeroed by the caller);
     overwrites ``grad_sampling_loc`` (…, 3) and ``grad_attn_weight``."""
     named = dict(value=value, value_dpt_dist=value_dpt_dist, spatial_shapes=value_spatial_shapes,
                  level_start_index=value_level_start_index, sampling_loc=sampling_locations,
@@ -270,6 +276,8 @@ def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_leve
                  grad_attn_weight=grad_attn_weight)
     if grad_depth_score is not None:
         named["grad_depth_score"] = grad_depth_score
+    if grad_weight_update is not None:
+        named["grad_weight_update"] = grad_weight_update
     _contig(**named)
     dev = _on_gpu(**named)
     B, S, M, C, D, L, Q, P = _fused_dims(value, value_dpt_dist, value_spatial_shapes, value_level_start_index,
@@ -280,6 +288,10 @@ def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_leve
     _expect(grad_output, "grad_output", dtype=value.dtype)
     if grad_depth_score is not None:
         _expect(grad_depth_score, "grad_depth_score", shape=(B, Q, M, L, P, 4), dtype=value.dtype)
+    if grad_weight_update is not None:
+        if grad_weight_update.numel() != B * Q * M:
+            raise RuntimeError(f"grad_weight_update has {grad_weight_update.numel()} elements, expected {B * Q * M}")
+        _expect(grad_weight_update, "grad_weight_update", dtype=aux)
     _expect(grad_value, "grad_value", shape=value.shape, dtype=aux)
     _expect(grad_value_dpt_dist, "grad_value_dpt_dist", shape=value_dpt_dist.shape, dtype=aux)
     _expect(grad_sampling_loc, "grad_sampling_loc", shape=(B, Q, M, L, P, 3), dtype=aux)
@@ -295,7 +307,8 @@ def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_leve
         rc = _lib.lib().dfa3d_fused_backward(
             _lib.ptr(value), _lib.ptr(value_dpt_dist), _lib.ptr(value_spatial_shapes),
             _lib.ptr(value_level_start_index), _lib.ptr(sampling_locations), _lib.ptr(attention_weights),
-            _lib.ptr(grad_output), _lib.ptr(grad_depth_score), _lib.ptr(grad_value), _lib.ptr(grad_value_dpt_dist),
-            _lib.ptr(grad_sampling_loc), _lib.ptr(grad_attn_weight), _lib.ptr(workspace), ws_bytes,
-            B, S, M, C, D, L, Q, P, code, _lib.stream_of(value))
+            _lib.ptr(grad_output), _lib.ptr(grad_depth_score), _lib.ptr(grad_weight_update), _lib.ptr(grad_value),
+            _lib.ptr(grad_value_dpt_dist), _lib.ptr(grad_sampling_loc), _lib.ptr(grad_attn_weight),
+            _lib.ptr(workspace), ws_bytes, B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2], code,
+            _lib.stream_of(value))
     _lib.check(rc, "dfa3d_fused_backward")

@@ -39,6 +39,7 @@ __all__ = [
     "MultiScale3DDeformableAttnFunction_fp32",
     "MultiScaleDepthScoreSampleFunction_fp16", "WeightedMultiScaleDeformableAttnFunction_fp16",
     "MultiScale3DDeformableAttnFunction_fp16",
+    "MultiScale3DDeformableAttnWeightUpdateFunction", "MultiScale3DDeformableAttnWeightUpdateFunction_fp32",
 ]
 
 
@@ -147,6 +148,49 @@ class MultiScale3DDeformableAttnFunction(Function):
             grad_sampling_loc, grad_attn_weight, None
 
 
+class MultiScale3DDeformableAttnWeightUpdateFunction(Function):
+    """One-stage DFA3D that returns ``(output, weight_update)`` instead of the depth scores:
+    ``weight_update`` (bs, Q, heads, 1) is the reduction the reference's caller applies to the score tensor,
+    ``(depth_score.mean(-1) * attention_weights).flatten(-2).sum(-1, keepdim=True)``
+    (BEVFormer_DFA3D/projects/mmdet3d_plugin/bevformer/modules/spatial_cross_attention.py:579), computed in the
+    kernel so that the (bs, Q, heads, L, P, 4) score tensor is never written.  ``value_dpt_dist`` may be
+    (bs, keys, 1, D): one distribution for all heads, without the repeat of spatial_cross_attention.py:496-497.
+    Both outputs are differentiable."""
+
+    @staticmethod
+    def forward(ctx, value, value_dpt_dist, value_spatial_shapes, value_level_start_index,
+                sampling_locations, attention_weights, im2col_step):
+        ctx.im2col_step = im2col_step
+        ctx.set_materialize_grads(False)
+        output, _, weight_update = _ext.dfa3d_fused_forward(
+            value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
+            attention_weights, im2col_step=ctx.im2col_step, need_depth_score=False, need_weight_update=True)
+        ctx.save_for_backward(value, value_dpt_dist, value_spatial_shapes, value_level_start_index,
+                              sampling_locations, attention_weights)
+        return output, weight_update.to(attention_weights.dtype)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_output, grad_weight_update):
+        value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations, \
+            attention_weights = ctx.saved_tensors
+        aux = _aux(value)
+        if grad_output is None:
+            grad_output = torch.zeros(value.shape[0], sampling_locations.shape[1], value.shape[2] * value.shape[3],
+                                      dtype=value.dtype, device=value.device)
+        grad_value = torch.zeros(value.shape, dtype=aux, device=value.device)
+        grad_value_dpt_dist = torch.zeros(value_dpt_dist.shape, dtype=aux, device=value.device)
+        grad_sampling_loc = torch.empty_like(sampling_locations)
+        grad_attn_weight = torch.empty_like(attention_weights)
+        _ext.dfa3d_fused_backward(
+            value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
+            attention_weights, _grad_in(grad_output, value.dtype), None,
+            grad_value, grad_value_dpt_dist, grad_sampling_loc, grad_attn_weight, im2col_step=ctx.im2col_step,
+            grad_weight_update=None if grad_weight_update is None else _grad_in(grad_weight_update, aux))
+        return grad_value.to(value.dtype), grad_value_dpt_dist.to(value_dpt_dist.dtype), None, None, \
+            grad_sampling_loc, grad_attn_weight, None
+
+
 def _autocast_twin(base, name, doc):
     """Subclass whose forward casts floating inputs to float32 under ``torch.autocast`` (what the
     reference's ``custom_fwd(cast_inputs=torch.float32)`` twins do) and runs outside autocast."""
@@ -182,3 +226,5 @@ WeightedMultiScaleDeformableAttnFunction_fp16 = _autocast_twin(
     WeightedMultiScaleDeformableAttnFunction, "WeightedMultiScaleDeformableAttnFunction_fp16", _FP16_DOC)
 MultiScale3DDeformableAttnFunction_fp16 = _autocast_twin(
     MultiScale3DDeformableAttnFunction, "MultiScale3DDeformableAttnFunction_fp16", _FP16_DOC)
+MultiScale3DDeformableAttnWeightUpdateFunction_fp32 = _autocast_twin(
+    MultiScale3DDeformableAttnWeightUpdateFunction, "MultiScale3DDeformableAttnWeightUpdateFunction_fp32", _FP32_DOC)

@@ -181,8 +181,8 @@ def main():
     def backward_call():
         _lib.check(L_.dfa3d_fused_backward(
             _lib.ptr(vd), _lib.ptr(dd), _lib.ptr(shapes), _lib.ptr(lsi), _lib.ptr(ld), _lib.ptr(ad), _lib.ptr(go), None,
-            _lib.ptr(gv), _lib.ptr(gd), _lib.ptr(gl), _lib.ptr(ga), _lib.ptr(ws) if ws_bytes else None, ws_bytes,
-            B, S, M, C, D, L, Q, P, code, stream), "dfa3d_fused_backward")
+            None, _lib.ptr(gv), _lib.ptr(gd), _lib.ptr(gl), _lib.ptr(ga), _lib.ptr(ws) if ws_bytes else None, ws_bytes,
+            B, S, M, C, D, L, Q, P, dist.shape[2], code, stream), "dfa3d_fused_backward")
 
     def zero():
         gv.zero_()

@@ -97,18 +97,27 @@ size_t dfa3d_wms_deform_attn_backward_workspace_bytes(int B, int S, int M, int C
 /* Both stages in one kernel: what the reference's one-stage autograd Function does with two
  * native calls and two slice copies
  * (BEVFormer_DFA3D/projects/mmdet3d_plugin/bevformer/modules/multi_scale_3ddeformable_attn_function.py:279-303).
- * Writes every element of `out` and, when `score` is not NULL, of `score`. */
+ * Writes every element of `out` and, when they are not NULL, of `score` (B,Q,M,L,P,4) and of
+ * `weight_update` (B,Q,M; float for DFA3D_F32 / DFA3D_BF16, double for DFA3D_F64).
+ *
+ * `dist_heads` is M for a distribution per head, dist (B,S,M,D), or 1 for one distribution shared by
+ * all heads, dist (B,S,1,D): what the reference's caller builds with an 8-fold repeat
+ * (BEVFormer_DFA3D/projects/mmdet3d_plugin/bevformer/modules/spatial_cross_attention.py:496-497).
+ * weight_update[b,q,m] = sum over (l,p) of attn * mean of the four corner scores: the reduction that
+ * caller applies to the score tensor right after the call (spatial_cross_attention.py:579). */
 int dfa3d_fused_forward(
     const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
     const void *loc3, const void *attn,
-    void *out, void *score,
-    int B, int S, int M, int C, int D, int L, int Q, int P, int dtype, void *stream);
+    void *out, void *score, void *weight_update,
+    int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype, void *stream);
 
 /* Backward of dfa3d_fused_forward (…_function.py:306-352: two native calls, six zero fills and
  * a host synchronisation in the reference).  The depth scores are recomputed from `dist`, not
- * read back.  `grad_score_in` (may be NULL) is an incoming gradient with respect to the `score`
- * output and is chained into grad_dist and the z gradient.  `grad_value` and `grad_dist` must be
- * zero on entry and hold the gradients on return; `grad_loc3` and `grad_attn` are overwritten.
+ * read back.  `grad_score_in` (B,Q,M,L,P,4) and `grad_weight_update` (B,Q,M; float / double as
+ * above), either of which may be NULL, are incoming gradients with respect to the `score` and
+ * `weight_update` outputs and are chained into grad_dist, grad_attn and the z gradient.
+ * `grad_value` (B,S,M,C) and `grad_dist` (B,S,dist_heads,D) must be zero on entry and hold the
+ * gradients on return; `grad_loc3` and `grad_attn` are overwritten.
  *
  * `workspace` (may be NULL) is caller-owned scratch device memory, 256-byte aligned, of at least
  * dfa3d_fused_backward_workspace_bytes(...) bytes, whose contents need not be preserved or
@@ -119,9 +128,10 @@ int dfa3d_fused_forward(
 int dfa3d_fused_backward(
     const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
     const void *loc3, const void *attn, const void *grad_out, const void *grad_score_in,
+    const void *grad_weight_update,
     void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn,
     void *workspace, size_t workspace_bytes,
-    int B, int S, int M, int C, int D, int L, int Q, int P, int dtype, void *stream);
+    int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype, void *stream);
 
 /* Scratch bytes dfa3d_fused_backward wants for these dimensions; 0 when the binned path does not
  * apply (DFA3D_F64, rows too long for LDS tiles, more than 2^31 points, invalid dimensions). */

@@ -165,6 +165,93 @@ def test_gradient_through_depth_score_output(oracle):
     _compare(got, want, dict(rtol=1e-10, atol=1e-11), dict(rtol=1e-10, atol=1e-11))
 
 
+def _shared_dist_expectation(oracle, inp, grad_wu=None):
+    """Checker results for a distribution shared by the heads: the checker sees the 8-fold repeat the
+    reference's caller makes (spatial_cross_attention.py:496-497) and its grad_dist is summed over heads;
+    a gradient at the weight_update output enters as a gradient of the scores and of the weights."""
+    M = inp["value"].shape[2]
+    rep = dict(inp)
+    rep["value_dpt_dist"] = inp["value_dpt_dist"].repeat(1, 1, M // inp["value_dpt_dist"].shape[2], 1).contiguous()
+    out, score, gv, gd, gl, ga = _oracle_one_stage(oracle, rep)
+    attn = inp["attention_weights"]
+    wu = (score.mean(-1) * attn).flatten(-2).sum(-1, keepdim=True)
+    if grad_wu is not None:
+        gsc = (grad_wu[..., None, None] * attn[..., None] / 4).expand_as(score).contiguous()
+        extra_gd, extra_gl = oracle.depth_score_backward(rep["value_dpt_dist"], inp["spatial_shapes"],
+                                                         inp["level_start_index"], inp["sampling_locations"], gsc)
+        gd = gd + extra_gd
+        gl = gl + extra_gl
+        ga = ga + grad_wu[..., None] * score.mean(-1)
+    if inp["value_dpt_dist"].shape[2] == 1:
+        gd = gd.sum(2, keepdim=True)
+    return out, score, wu, gv, gd, gl, ga
+
+
+@pytest.mark.parametrize("case", [TINY[0], TINY[1], TINY[3], TINY[4]], ids=lambda c: f"seed{c['seed']}")
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32], ids=["fp64", "fp32"])
+def test_shared_distribution_and_weight_update(oracle, case, dtype):
+    """dist (B,S,1,D) used by every head, with the score tensor and with the fused weight_update output
+    (gradients arriving at both outputs), against the checker on the repeated distribution.  fp64 runs the
+    kernels with device-memory atomics, fp32 the LDS-tile kernels."""
+    from dfa3D.functional import MultiScale3DDeformableAttnFunction, MultiScale3DDeformableAttnWeightUpdateFunction
+    dev = _dev()
+    t = tiny_case(**case)
+    inp = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in _as_inputs(t).items()}
+    inp["value_dpt_dist"] = inp["value_dpt_dist"][:, :, :1].contiguous()
+    g = torch.Generator().manual_seed(77)
+    grad_wu = torch.randn(*inp["attention_weights"].shape[:3], 1, generator=g, dtype=dtype)
+    fwd_tol, bwd_tol = (dict(rtol=1e-10, atol=1e-11),) * 2 if dtype == torch.float64 else (F32_FWD, F32_BWD)
+
+    def leaves():
+        return [inp[k].to(dev).requires_grad_() for k in ("value", "value_dpt_dist", "sampling_locations",
+                                                          "attention_weights")]
+    shapes3, lsi, go = inp["spatial_shapes"].to(dev), inp["level_start_index"].to(dev), inp["grad_output"].to(dev)
+
+    # (output, depth_score) with the shared distribution
+    want = _shared_dist_expectation(oracle, inp)
+    v, d, loc, a = leaves()
+    out, score = MultiScale3DDeformableAttnFunction.apply(v, d, shapes3, lsi, loc, a, 64)
+    grads = torch.autograd.grad(out, [v, d, loc, a], go)
+    got = [x.detach().cpu() for x in (out, score, *grads)]
+    _compare(got, [want[0], want[1], *want[3:]], fwd_tol, bwd_tol)
+
+    # (output, weight_update), gradients at both
+    want = _shared_dist_expectation(oracle, inp, grad_wu=grad_wu)
+    v, d, loc, a = leaves()
+    out, wu = MultiScale3DDeformableAttnWeightUpdateFunction.apply(v, d, shapes3, lsi, loc, a, 64)
+    grads = torch.autograd.grad([out, wu], [v, d, loc, a], [go, grad_wu.to(dev)])
+    torch.testing.assert_close(wu.detach().cpu(), want[2], **fwd_tol)
+    got = [x.detach().cpu() for x in (out, score, *grads)]
+    _compare(got, [want[0], want[1], *want[3:]], fwd_tol, bwd_tol)
+
+    # weight_update with a distribution per head, gradient at weight_update alone
+    inp_m = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in _as_inputs(t).items()}
+    want = _shared_dist_expectation(oracle, inp_m, grad_wu=grad_wu)
+    v, d, loc, a = [inp_m[k].to(dev).requires_grad_() for k in ("value", "value_dpt_dist", "sampling_locations",
+                                                                 "attention_weights")]
+    out, wu = MultiScale3DDeformableAttnWeightUpdateFunction.apply(v, d, shapes3, lsi, loc, a, 64)
+    grads = torch.autograd.grad([out, wu], [v, d, loc, a], [go, grad_wu.to(dev)])
+    torch.testing.assert_close(wu.detach().cpu(), want[2], **fwd_tol)
+    _compare([out.detach().cpu(), want[1], *[x.cpu() for x in grads]], [want[0], want[1], *want[3:]], fwd_tol, bwd_tol)
+
+
+def test_fp32_base_shape_shared_distribution_weight_update(oracle):
+    """BEVFormer-base shape as its caller has it: one distribution for the 8 heads, weight_update wanted."""
+    from dfa3D.functional import MultiScale3DDeformableAttnWeightUpdateFunction
+    from dfa3D.workloads import WORKLOADS, make_inputs
+    dev = _dev()
+    inp = make_inputs(WORKLOADS["base"])
+    inp["value_dpt_dist"] = inp["value_dpt_dist"][:, :, :1].contiguous()
+    want = _shared_dist_expectation(oracle, inp)
+    v, d, loc, a = [inp[k].to(dev).requires_grad_() for k in ("value", "value_dpt_dist", "sampling_locations",
+                                                               "attention_weights")]
+    out, wu = MultiScale3DDeformableAttnWeightUpdateFunction.apply(
+        v, d, inp["spatial_shapes"].to(dev), inp["level_start_index"].to(dev), loc, a, 64)
+    grads = torch.autograd.grad(out, [v, d, loc, a], inp["grad_output"].to(dev))
+    torch.testing.assert_close(wu.detach().cpu(), want[2], **F32_FWD)
+    _compare([out.detach().cpu(), want[1], *[x.cpu() for x in grads]], [want[0], want[1], *want[3:]], F32_FWD, F32_BWD)
+
+
 @pytest.mark.parametrize("name", ["unit", "small"])
 def test_fp32_workloads_match_checker(oracle, name):
     from dfa3D.workloads import WORKLOADS, make_inputs

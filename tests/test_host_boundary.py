@@ -37,20 +37,23 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     null = ctypes.c_void_p(0)
     one = ctypes.c_void_p(256)          # never dereferenced: validation fails first
     # non-positive dimension
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, 0, 10, 8, 32, 16, 2, 5, 4, 0, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 0, 10, 8, 32, 16, 2, 5, 4, 8, 0, null)
     assert rc == -1 and b"positive" in L.dfa3d_last_error()
     # unknown dtype
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, 1, 10, 8, 32, 16, 2, 5, 4, 7, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 7, null)
     assert rc == -1 and b"dtype" in L.dfa3d_last_error()
     # too many levels
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, 1, 10, 8, 32, 16, 17, 5, 4, 0, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 17, 5, 4, 8, 0, null)
     assert rc == -2 and b"levels" in L.dfa3d_last_error()
     # a batch element beyond 2^30 bytes
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, 1, 1 << 20, 8, 64, 16, 2, 5, 4, 0, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 1 << 20, 8, 64, 16, 2, 5, 4, 8, 0, null)
     assert rc == -2 and b"2^30" in L.dfa3d_last_error()
     # NULL operand
-    rc = L.dfa3d_fused_forward(null, one, one, one, one, one, one, one, 1, 10, 8, 32, 16, 2, 5, 4, 0, null)
+    rc = L.dfa3d_fused_forward(null, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 0, null)
     assert rc == -1 and b"NULL" in L.dfa3d_last_error()
+    # a distribution for 3 of the 8 heads
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 3, 0, null)
+    assert rc == -1 and b"dist_heads" in L.dfa3d_last_error()
     rc = L.dfa3d_wms_deform_attn_forward(one, one, 4, one, one, 2, one, one, one, 1, 10, 8, 32, 2, 5, 4, 0, null)
     assert rc == -1 and b"stride" in L.dfa3d_last_error()
     rc = L.dfa3d_ms_depth_score_sample_backward(one, one, one, one, one, null, one, null, 0, 1, 10, 8, 16, 2, 5, 4, 0, null)
