@@ -193,7 +193,7 @@ int dfa3d_wms_deform_attn_forward(const void *value, const int64_t *shapes, int 
   if (shape_stride < 2 || shape_stride > 3 || loc_stride < 2 || loc_stride > 3)
     return fail(DFA3D_EINVAL, "%s: shape_stride and loc_stride must be 2 or 3", fn);
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, shapes); REQUIRE_PTR(fn, level_start); REQUIRE_PTR(fn, loc);
-  REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, score); REQUIRE_PTR(fn, out);
+  REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, out);                  // score == NULL: every score is 1
   dfa3d::FwdArgs a{};
   a.value = value; a.dist = nullptr; a.shapes = shapes; a.shape_stride = shape_stride; a.level_start = level_start;
   a.loc = loc; a.loc_stride = loc_stride; a.attn = attn; a.score_in = score; a.out = out; a.score_out = nullptr;
@@ -241,8 +241,9 @@ int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int
       grad_loc_stride > 3)
     return fail(DFA3D_EINVAL, "%s: shape_stride, loc_stride and grad_loc_stride must be 2 or 3", fn);
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, shapes); REQUIRE_PTR(fn, level_start); REQUIRE_PTR(fn, loc);
-  REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, score); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
-  REQUIRE_PTR(fn, grad_loc); REQUIRE_PTR(fn, grad_attn); REQUIRE_PTR(fn, grad_score);
+  REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
+  REQUIRE_PTR(fn, grad_loc); REQUIRE_PTR(fn, grad_attn);
+  if (score != nullptr) REQUIRE_PTR(fn, grad_score);            // score == NULL: every score is 1, no gradient for it
   const dfa3d::BwdArgs a = wms_bwd_args(value, shapes, shape_stride, level_start, loc, loc_stride, attn, score,
                                         grad_out, grad_value, grad_loc, grad_loc_stride, grad_attn, grad_score, B, S,
                                         M, C, L, Q, P);

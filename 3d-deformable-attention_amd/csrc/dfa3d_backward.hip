@@ -186,7 +186,7 @@ __global__ __launch_bounds__(kBlock) void bwd_attention_kernel(
         } else {
           const T *si = score_in + gp * 4;
 #pragma unroll
-          for (int k = 0; k < 4; ++k) sc[k] = Elem<T>::ld(si + k);
+          for (int k = 0; k < 4; ++k) sc[k] = score_in != nullptr ? Elem<T>::ld(si + k) : (A)1;
         }
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -270,7 +270,7 @@ __global__ __launch_bounds__(kBlock) void bwd_attention_kernel(
             gz += (g.key[k] >= 0 && tap.inside) ? gs[k] * (hi[k] - lo[k]) : (A)0;
           }
           gl[2] = gz * (A)tab.Dd[l];
-        } else {
+        } else if (grad_score_out != nullptr) {
           A *go4 = grad_score_out + gp * 4;
 #pragma unroll
           for (int k = 0; k < 4; ++k) go4[k] = gs[k];

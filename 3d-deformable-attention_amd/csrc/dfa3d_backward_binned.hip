@@ -396,7 +396,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         } else {
           const T *si = score_in + gp * 4;
 #pragma unroll
-          for (int k = 0; k < 4; ++k) sc[k] = Elem<T>::ld(si + k);
+          for (int k = 0; k < 4; ++k) sc[k] = score_in != nullptr ? Elem<T>::ld(si + k) : 1.f;
         }
         my_goff = (uint32_t)((unit - (size_t)b * Q * M) * C * sizeof(T));
 #pragma unroll
@@ -577,7 +577,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
             gz += (g.key[k] >= 0 && tap.inside) ? gs[k] * (hi[k] - lo[k]) : 0.f;
           }
           gl[2] = gz * (float)Dd;
-        } else {
+        } else if (grad_score_out != nullptr) {
           float *go4 = grad_score_out + gp * 4;
 #pragma unroll
           for (int k = 0; k < 4; ++k) go4[k] = gs[k];

@@ -119,9 +119,9 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
             }
             wu = a * ((sc[0] + sc[1] + sc[2] + sc[3]) * (A)0.25);
           } else {
-            const T *si = score_in + gp * 4;
+            const T *si = score_in + gp * 4;        // no scores given: plain deformable attention
 #pragma unroll
-            for (int k = 0; k < 4; ++k) sc[k] = Elem<T>::ld(si + k);
+            for (int k = 0; k < 4; ++k) sc[k] = score_in != nullptr ? Elem<T>::ld(si + k) : (A)1;
           }
 #pragma unroll
           for (int k = 0; k < 4; ++k) {

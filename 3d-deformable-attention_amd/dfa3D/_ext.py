@@ -218,6 +218,65 @@ def wms_deform_attn_backward(value, value_spatial_shapes, value_level_start_inde
     _lib.check(rc, "dfa3d_wms_deform_attn_backward")
 
 
+def ms_deform_attn_forward(value, value_spatial_shapes, value_level_start_index, sampling_locations,
+                           attention_weights, im2col_step):
+    """Plain multi-scale deformable attention (every depth score 1): the entry point BEVFormer's temporal
+    self-attention and decoder load from mmcv's extension
+    (BEVFormer_DFA3D/projects/mmdet3d_plugin/bevformer/modules/multi_scale_deformable_attn_function.py:10-12,:47-53).
+    Runs the stage-2 kernel without a score tensor."""
+    named = dict(value=value, spatial_shapes=value_spatial_shapes, level_start_index=value_level_start_index,
+                 sampling_loc=sampling_locations, attn_weight=attention_weights)
+    _contig(**named)
+    dev = _on_gpu(**named)
+    B, S, M, C, L, Q, P, sw, lw = _wms_dims(value, value_spatial_shapes, value_level_start_index, sampling_locations,
+                                            attention_weights, None, "ms_deform_attn_forward")
+    _step(B, im2col_step)
+    out = torch.empty(B, Q, M * C, dtype=value.dtype, device=dev)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(dev):
+        rc = _lib.lib().dfa3d_wms_deform_attn_forward(
+            _lib.ptr(value), _lib.ptr(value_spatial_shapes), sw, _lib.ptr(value_level_start_index),
+            _lib.ptr(sampling_locations), lw, _lib.ptr(attention_weights), None, _lib.ptr(out),
+            B, S, M, C, L, Q, P, _lib.dtype_code(value), _lib.stream_of(value))
+    _lib.check(rc, "dfa3d_wms_deform_attn_forward")
+    return out
+
+
+def ms_deform_attn_backward(value, value_spatial_shapes, value_level_start_index, sampling_locations,
+                            attention_weights, grad_output, grad_value, grad_sampling_loc, grad_attn_weight,
+                            im2col_step):
+    """Backward of ms_deform_attn_forward (…/multi_scale_deformable_attn_function.py:74-84).  Accumulates into
+    ``grad_value`` (pre-zeroed by the caller); overwrites ``grad_sampling_loc`` and ``grad_attn_weight``."""
+    named = dict(value=value, spatial_shapes=value_spatial_shapes, level_start_index=value_level_start_index,
+                 sampling_loc=sampling_locations, attn_weight=attention_weights, grad_output=grad_output,
+                 grad_value=grad_value, grad_sampling_loc=grad_sampling_loc, grad_attn_weight=grad_attn_weight)
+    _contig(**named)
+    dev = _on_gpu(**named)
+    B, S, M, C, L, Q, P, sw, lw = _wms_dims(value, value_spatial_shapes, value_level_start_index, sampling_locations,
+                                            attention_weights, None, "ms_deform_attn_backward")
+    aux = _aux_dtype(value.dtype)
+    if grad_output.numel() != B * Q * M * C:
+        raise RuntimeError(f"grad_output has {grad_output.numel()} elements, expected {B * Q * M * C}")
+    _expect(grad_output, "grad_output", dtype=value.dtype)
+    _expect(grad_value, "grad_value", shape=value.shape, dtype=aux)
+    _expect(grad_sampling_loc, "grad_sampling_loc", shape=sampling_locations.shape, dtype=aux)
+    _expect(grad_attn_weight, "grad_attn_weight", shape=(B, Q, M, L, P), dtype=aux)
+    _step(B, im2col_step)
+    if grad_output.numel() == 0:
+        return
+    code = _lib.dtype_code(value)
+    ws_bytes = _lib.lib().dfa3d_wms_deform_attn_backward_workspace_bytes(B, S, M, C, L, Q, P, code)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
+    with torch.cuda.device(dev):
+        rc = _lib.lib().dfa3d_wms_deform_attn_backward(
+            _lib.ptr(value), _lib.ptr(value_spatial_shapes), sw, _lib.ptr(value_level_start_index),
+            _lib.ptr(sampling_locations), lw, _lib.ptr(attention_weights), None, _lib.ptr(grad_output),
+            _lib.ptr(grad_value), _lib.ptr(grad_sampling_loc), lw, _lib.ptr(grad_attn_weight), None,
+            _lib.ptr(workspace), ws_bytes, B, S, M, C, L, Q, P, code, _lib.stream_of(value))
+    _lib.check(rc, "dfa3d_wms_deform_attn_backward")
+
+
 def _fused_dims(value, dist, shapes3, lsi, loc3, attn, name):
     if value.dim() != 4 or dist.dim() != 4 or value.shape[:2] != dist.shape[:2] or \
             dist.shape[2] not in (1, value.shape[2]):

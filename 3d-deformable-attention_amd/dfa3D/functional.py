@@ -40,6 +40,7 @@ __all__ = [
     "MultiScaleDepthScoreSampleFunction_fp16", "WeightedMultiScaleDeformableAttnFunction_fp16",
     "MultiScale3DDeformableAttnFunction_fp16",
     "MultiScale3DDeformableAttnWeightUpdateFunction", "MultiScale3DDeformableAttnWeightUpdateFunction_fp32",
+    "MultiScaleDeformableAttnFunction", "MultiScaleDeformableAttnFunction_fp32", "MultiScaleDeformableAttnFunction_fp16",
 ]
 
 
@@ -109,6 +110,38 @@ class WeightedMultiScaleDeformableAttnFunction(Function):
             grad_depth_score, im2col_step=ctx.im2col_step)
         return grad_value.to(value.dtype), None, None, grad_sampling_loc, grad_attn_weight, \
             grad_depth_score.to(depth_score.dtype), None
+
+
+class MultiScaleDeformableAttnFunction(Function):
+    """Plain (2-D) multi-scale deformable attention: stage 2 with every depth score equal to 1.  Same signature
+    as the Function BEVFormer's temporal self-attention and decoder cross-attention use
+    (BEVFormer_DFA3D/projects/mmdet3d_plugin/bevformer/modules/multi_scale_deformable_attn_function.py:90-163)."""
+
+    @staticmethod
+    def forward(ctx, value, value_spatial_shapes, value_level_start_index, sampling_locations,
+                attention_weights, im2col_step):
+        ctx.im2col_step = im2col_step
+        output = _ext.ms_deform_attn_forward(value, value_spatial_shapes, value_level_start_index,
+                                             sampling_locations, attention_weights, im2col_step=ctx.im2col_step)
+        ctx.save_for_backward(value, value_spatial_shapes, value_level_start_index, sampling_locations,
+                              attention_weights)
+        return output
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_output):
+        value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights = \
+            ctx.saved_tensors
+        grad_value = torch.zeros(value.shape, dtype=_aux(value), device=value.device)
+        grad_sampling_loc = torch.empty_like(sampling_locations)
+        if sampling_locations.shape[-1] > 2:
+            grad_sampling_loc[..., 2:] = 0
+        grad_attn_weight = torch.empty_like(attention_weights)
+        _ext.ms_deform_attn_backward(
+            value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights,
+            _grad_in(grad_output, value.dtype), grad_value, grad_sampling_loc, grad_attn_weight,
+            im2col_step=ctx.im2col_step)
+        return grad_value.to(value.dtype), None, None, grad_sampling_loc, grad_attn_weight, None
 
 
 class MultiScale3DDeformableAttnFunction(Function):
@@ -228,3 +261,7 @@ MultiScale3DDeformableAttnFunction_fp16 = _autocast_twin(
     MultiScale3DDeformableAttnFunction, "MultiScale3DDeformableAttnFunction_fp16", _FP16_DOC)
 MultiScale3DDeformableAttnWeightUpdateFunction_fp32 = _autocast_twin(
     MultiScale3DDeformableAttnWeightUpdateFunction, "MultiScale3DDeformableAttnWeightUpdateFunction_fp32", _FP32_DOC)
+MultiScaleDeformableAttnFunction_fp32 = _autocast_twin(
+    MultiScaleDeformableAttnFunction, "MultiScaleDeformableAttnFunction_fp32", _FP32_DOC)
+MultiScaleDeformableAttnFunction_fp16 = _autocast_twin(
+    MultiScaleDeformableAttnFunction, "MultiScaleDeformableAttnFunction_fp16", _FP16_DOC)

@@ -1,0 +1,3 @@
+from .ms_deform_attn_3d import MSDeformableAttention3D_DFA3D
+
+__all__ = ["MSDeformableAttention3D_DFA3D"]

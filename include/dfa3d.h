@@ -72,7 +72,10 @@ size_t dfa3d_ms_depth_score_sample_backward_workspace_bytes(int B, int S, int M,
                                                             int dtype);
 
 /* Stage 2 forward: depth-weighted multi-scale deformable attention.  Writes every element of
- * `out`.  Replaces wms_deform_attn_forward
+ * `out`.  `score` == NULL stands for scores that are all 1: plain multi-scale deformable attention,
+ * mmcv's ms_deform_attn_forward as BEVFormer's other attention layers call it
+ * (BEVFormer_DFA3D/projects/mmdet3d_plugin/bevformer/modules/multi_scale_deformable_attn_function.py:47-53).
+ * Replaces wms_deform_attn_forward
  * (pybind.cpp:43-47 -> DFA3D/dfa3D/ops/csrc/cuda/wms_deform_attn_cuda.cu:213-288). */
 int dfa3d_wms_deform_attn_forward(
     const void *value, const int64_t *shapes, int shape_stride, const int64_t *level_start,
@@ -82,7 +85,8 @@ int dfa3d_wms_deform_attn_forward(
 
 /* Stage 2 backward.  `grad_value` must be zero on entry and holds the gradient on return;
  * `grad_loc` (B,Q,M,L,P,grad_loc_stride) gets its first two components overwritten, `grad_attn` and
- * `grad_score` are overwritten.  `workspace` as for dfa3d_fused_backward (size from
+ * `grad_score` are overwritten (`score` == NULL: scores all 1, `grad_score` may be NULL and is then not
+ * written).  `workspace` as for dfa3d_fused_backward (size from
  * dfa3d_wms_deform_attn_backward_workspace_bytes; NULL = device-memory atomics).
  * Replaces wms_deform_attn_backward
  * (pybind.cpp:48-54 -> wms_deform_attn_cuda.cu:291-370). */

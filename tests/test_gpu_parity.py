@@ -165,6 +165,32 @@ def test_gradient_through_depth_score_output(oracle):
     _compare(got, want, dict(rtol=1e-10, atol=1e-11), dict(rtol=1e-10, atol=1e-11))
 
 
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32], ids=["fp64", "fp32"])
+@pytest.mark.parametrize("width", [2, 3])
+def test_plain_deformable_attention_matches_grid_sample(oracle, dtype, width):
+    """MultiScaleDeformableAttnFunction (no depth scores) against multi-scale deformable attention written
+    with 2-D grid_sample and differentiated by autograd, and against the checker's stage 2 with scores of 1."""
+    from forms import msda_2d_form
+    from dfa3D.functional import MultiScaleDeformableAttnFunction
+    dev = _dev()
+    t = tiny_case(21, C=32, M=4, Q=9, P=4, levels=((6, 9), (4, 5), (3, 3)), dtype=dtype)
+    shapes = t["shapes3"][:, :width].contiguous()
+    loc = t["loc"][..., :width].contiguous()
+    cpu = [x.clone().requires_grad_() for x in (t["value"], loc, t["attn"])]
+    want = msda_2d_form(cpu[0], t["levels"], cpu[1][..., :2], cpu[2])
+    want_grads = torch.autograd.grad(want, cpu, t["grad_out"])
+    gpu = [x.to(dev).requires_grad_() for x in (t["value"], loc, t["attn"])]
+    out = MultiScaleDeformableAttnFunction.apply(gpu[0], shapes.to(dev), t["lsi"].to(dev), gpu[1], gpu[2], 64)
+    grads = torch.autograd.grad(out, gpu, t["grad_out"].to(dev))
+    fwd_tol, bwd_tol = (dict(rtol=1e-10, atol=1e-11),) * 2 if dtype == torch.float64 else (F32_FWD, F32_BWD)
+    torch.testing.assert_close(out.detach().cpu(), want.detach(), **fwd_tol)
+    for g, w in zip(grads, want_grads):
+        torch.testing.assert_close(g.cpu(), w, **bwd_tol)
+    ones = torch.ones(*t["attn"].shape, 4, dtype=dtype)
+    torch.testing.assert_close(out.detach().cpu(), oracle.wms_forward(
+        t["value"], t["shapes3"][:, :2].contiguous(), t["lsi"], t["loc"][..., :2].contiguous(), t["attn"], ones), **fwd_tol)
+
+
 def _shared_dist_expectation(oracle, inp, grad_wu=None):
     """Checker results for a distribution shared by the heads: the checker sees the 8-fold repeat the
     reference's caller makes (spatial_cross_attention.py:496-497) and its grad_dist is summed over heads;
