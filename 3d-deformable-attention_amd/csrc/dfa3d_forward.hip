@@ -190,8 +190,11 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
-// Stage 1 alone: one lane per sampling point, grid-stride over all B*Q*M*L*P points.
+// Stage 1 alone: one lane per sampling point.  Block id -> (head, batch, block of kDsQueries
+// queries) with head = block % M, as in the attention kernels: the distributions one XCD's L2
+// sees are those of one head.
 // ---------------------------------------------------------------------------------------
+constexpr int kDsQueries = 32;
 template <typename T, typename A>
 __global__ __launch_bounds__(kBlock) void depth_score_kernel(
     const T *__restrict__ dist, const int64_t *__restrict__ shapes3, const int64_t *__restrict__ level_start,
@@ -199,18 +202,20 @@ __global__ __launch_bounds__(kBlock) void depth_score_kernel(
   __shared__ LevelTable tab;
   load_level_table(tab, shapes3, 3, level_start, L, S, D);
   const int LP = L * P;
-  const size_t n = (size_t)B * Q * M * LP;
-  for (size_t gp = (size_t)blockIdx.x * kBlock + threadIdx.x; gp < n; gp += (size_t)gridDim.x * kBlock) {
-    const int lp = (int)(gp % LP);
-    const size_t unit = gp / LP;
-    const int m = (int)(unit % M);
-    const int b = (int)(unit / M / Q);
+  const int m = blockIdx.x % M;
+  const int rest = blockIdx.x / M;
+  const int q_blocks = (Q + kDsQueries - 1) / kDsQueries;
+  const int qb = rest % q_blocks, b = rest / q_blocks;
+  const int q0 = qb * kDsQueries, nq = min(kDsQueries, Q - q0);
+  const rsrc_t dist_r = make_rsrc(dist + (size_t)b * S * M * D, (size_t)S * M * D * sizeof(T));
+  for (int i = threadIdx.x; i < nq * LP; i += kBlock) {
+    const int ql = i / LP, lp = i - ql * LP;
+    const size_t gp = (((size_t)b * Q + q0 + ql) * M + m) * LP + lp;
     const int l = lp / P;
     const A *pl = loc3 + gp * 3;
     const Point2D<A> g = locate_2d<A>(pl[0], pl[1], tab.H[l], tab.W[l], tab.start[l]);
     const DepthTap<A> tap = locate_depth<A>(pl[2], tab.Dd[l]);
     A sc[4], lo[4], hi[4];
-    const rsrc_t dist_r = make_rsrc(dist + (size_t)b * S * M * D, (size_t)S * M * D * sizeof(T));
     corner_scores<T, A>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
     T *so = score + gp * 4;
 #pragma unroll
@@ -265,9 +270,8 @@ hipError_t launch_forward(const FwdArgs &a, int dtype, hipStream_t stream) {
 
 template <typename T, typename A>
 static hipError_t launch_ds_typed(const DepthScoreArgs &a, hipStream_t stream) {
-  const size_t n = (size_t)a.B * a.Q * a.M * a.L * a.P;
-  size_t blocks = (n + kBlock - 1) / kBlock;
-  if (blocks > (1u << 20)) blocks = 1u << 20;
+  const long long blocks = (long long)a.M * a.B * ((a.Q + kDsQueries - 1) / kDsQueries);
+  if (blocks <= 0 || blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
   hipLaunchKernelGGL((depth_score_kernel<T, A>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, (const T *)a.dist,
                      a.shapes3, a.level_start, (const A *)a.loc3, (T *)a.score, a.B, a.S, a.M, a.D, a.L, a.Q, a.P);
   return hipGetLastError();

@@ -47,8 +47,59 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain streaming copy of this many MiB (yardstick for profiler HBM counters)")
+    ap.add_argument("--no-variants", dest="variants", action="store_false",
+                    help="skip the timings of the two-stage, shared-distribution and plain-attention entry points")
     ap.add_argument("--tunable", action="append", default=[], metavar="NAME=VALUE", help="library launch tunable")
     return ap.parse_args()
+
+
+def variant_timings(_ext, torch, value, dist, shapes, lsi, loc, attn, go, reps):
+    """Event timings (ms, average) of the other entry points on the same operands: the reference's two-stage
+    composition, the caller-shaped call (one distribution for all heads, weight_update instead of the score
+    tensor) and plain multi-scale deformable attention (no depth scores)."""
+    dev = value.device
+    f32 = torch.float32
+    out = {}
+    score = _ext.ms_depth_score_sample_forward(dist, shapes, lsi, loc, 64)
+    gv = torch.zeros(value.shape, dtype=f32, device=dev)
+    gd = torch.zeros(dist.shape, dtype=f32, device=dev)
+    gl, gl3, ga = torch.empty_like(loc), torch.empty_like(loc), torch.empty_like(attn)
+    gs = torch.empty(score.shape, dtype=f32, device=dev)
+
+    def two_stage_fwd():
+        sc = _ext.ms_depth_score_sample_forward(dist, shapes, lsi, loc, 64)
+        _ext.wms_deform_attn_forward(value, shapes, lsi, loc, attn, sc, 64)
+
+    def two_stage_bwd():
+        gv.zero_()
+        gd.zero_()
+        _ext.wms_deform_attn_backward(value, shapes, lsi, loc, attn, score, go, gv, gl, ga, gs, 64)
+        _ext.ms_depth_score_sample_backward(dist, shapes, lsi, loc, gs.to(score.dtype), gd, gl3, 64)
+
+    out["two_stage_fwd_ms"] = round(event_time(two_stage_fwd, reps)[0], 4)
+    out["two_stage_bwd_ms"] = round(event_time(two_stage_bwd, reps)[0], 4)
+    del score, gs, gl3
+
+    shared = dist[:, :, :1].contiguous()
+    gd1 = torch.zeros(shared.shape, dtype=f32, device=dev)
+
+    def shared_bwd():
+        gv.zero_()
+        gd1.zero_()
+        _ext.dfa3d_fused_backward(value, shared, shapes, lsi, loc, attn, go, None, gv, gd1, gl, ga, 64)
+
+    out["shared_dist_weight_update_fwd_ms"] = round(event_time(lambda: _ext.dfa3d_fused_forward(
+        value, shared, shapes, lsi, loc, attn, 64, need_depth_score=False, need_weight_update=True), reps)[0], 4)
+    out["shared_dist_bwd_ms"] = round(event_time(shared_bwd, reps)[0], 4)
+
+    def plain_bwd():
+        gv.zero_()
+        _ext.ms_deform_attn_backward(value, shapes, lsi, loc, attn, go, gv, gl, ga, 64)
+
+    out["plain_msda_fwd_ms"] = round(event_time(lambda: _ext.ms_deform_attn_forward(value, shapes, lsi, loc, attn, 64),
+                                                reps)[0], 4)
+    out["plain_msda_bwd_ms"] = round(event_time(plain_bwd, reps)[0], 4)
+    return out
 
 
 def event_time(fn, reps, prep=None):
@@ -241,6 +292,8 @@ def main():
         "kernels": kernels,
         "roofline": roofline,
     }
+    if a.variants:
+        result["variants"] = variant_timings(_ext, torch, vd, dd, shapes, lsi, ld, ad, go, max(a.kernel_reps // 2, 3))
     if a.cpu_seconds > 0:
         result["cpu_baseline"] = cpu_baseline(w, a.cpu_seconds)
     print(json.dumps(result))
