@@ -26,7 +26,9 @@
 
 namespace dfa3d {
 
-constexpr int kQueues = 1;          // work-queue counters in the workspace
+constexpr int kClasses = 8;         // work queues: one per XCD (workgroup id % 8 with round-robin placement)
+constexpr int kQueueStride = 16;    // ints between queue counters: one 64-byte line each
+constexpr int kQueueInts = kClasses * kQueueStride + 32;   // + room for the optional phase timers
 constexpr int kBinQueries = 64;     // queries of one (batch, head) handled by a count/fill block
 constexpr int kHistCap = 8192;      // bins of one (batch, head) that fit the LDS histogram
 
@@ -34,15 +36,32 @@ struct BinPlan {
   int H[DFA3D_MAX_LEVELS], W[DFA3D_MAX_LEVELS], Dd[DFA3D_MAX_LEVELS], start[DFA3D_MAX_LEVELS];
   int tiles_x[DFA3D_MAX_LEVELS], level_base[DFA3D_MAX_LEVELS];
   int bins_per_bm;     // tiles over all levels of one (batch, head)
-  int total_bins;      // B * M * bins_per_bm
+  int total_bins;      // slots * bins_per_bm
+  int bins_per_class;  // total_bins / kClasses
+  int class_start[kClasses + 1];   // first work item of each head class (written by the scan)
   int ty, tx;          // tile edge in pixels
   int chunk;           // points of a bin handled by one work item
   int total_chunks;    // work items (written by the scan)
 };
 
+// Bins are numbered slot * bins_per_bm + tile, where the slot of (batch b, head m) puts the heads with the
+// same m % 8 next to each other: class c = m % 8 owns the slots [c, c + 1) * head_groups(M) * B.  The
+// binning blocks and the tile workgroups of class c run on XCD c, so everything written and read for one
+// head (records, gradients per point, tiles) goes through one L2.
+__host__ __device__ inline int head_groups(int M) { return (M + kClasses - 1) / kClasses; }
+__host__ __device__ inline int slot_count(int B, int M) { return kClasses * head_groups(M) * B; }
+__device__ __forceinline__ int slot_of(int b, int m, int B, int M) {
+  return ((m % kClasses) * head_groups(M) + m / kClasses) * B + b;
+}
+__device__ __forceinline__ void slot_decode(int slot, int B, int M, int &b, int &m) {
+  b = slot % B;
+  const int hm = slot / B, G = head_groups(M);
+  m = (hm % G) * kClasses + hm / G;
+}
+
 struct BinWorkspace {      // device pointers into the caller's workspace
   BinPlan *plan;
-  int *queues;             // kQueues counters
+  int *queues;             // kClasses counters, kQueueStride ints apart
   int *counts;             // points per bin
   int *cursor;             // begin of each bin's segment after the scan, end after the fill
   int *chunk_end;          // inclusive prefix of work items per bin
@@ -77,17 +96,19 @@ __global__ __launch_bounds__(256) void plan_and_clear_kernel(
     // the host sized the counters from an upper bound of the tile count; never exceed it
     if (base > max_bins_per_bm) base = 0;
     p.bins_per_bm = base;
-    p.total_bins = base * B * M;
+    p.total_bins = base * slot_count(B, M);
+    p.bins_per_class = base * head_groups(M) * B;
+    for (int c = 0; c <= kClasses; ++c) p.class_start[c] = 0;
     p.ty = ty; p.tx = tx;
     p.chunk = chunk; p.total_chunks = 0;
     *ws.plan = p;
   }
-  const size_t n = (size_t)max_bins_per_bm * B * M;
+  const size_t n = (size_t)max_bins_per_bm * slot_count(B, M);
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
     ws.counts[i] = 0;
     ws.cursor[i] = 0;
   }
-  if (blockIdx.x == 0 && threadIdx.x < 64) ws.queues[threadIdx.x] = 0;    // the counters and their padding
+  if (blockIdx.x == 0 && threadIdx.x < kQueueInts) ws.queues[threadIdx.x] = 0;    // the counters and their padding
 }
 
 // bin (within one (batch, head)) of a point that the operator does not skip
@@ -107,8 +128,11 @@ __global__ __launch_bounds__(256) void bin_points_kernel(
   const int nb = p.bins_per_bm;
   if (nb == 0) return;
   const bool use_lds = nb <= hist_cap;
-  const int bm = blockIdx.x / q_blocks, qb = blockIdx.x - bm * q_blocks;
-  const int b = bm / M, m = bm - b * M;
+  // head = block % M: with the round-robin placement of workgroups on the 8 XCDs, the records of one
+  // (batch, head) are written through one XCD's L2, which merges them into whole lines
+  const int m = blockIdx.x % M, rest = blockIdx.x / M;
+  const int qb = rest % q_blocks, b = rest / q_blocks;
+  const int bm = slot_of(b, m, B, M);
   const int LP = L * P;
   const int q0 = qb * kBinQueries, nq = min(kBinQueries, Q - q0);
   const int npts = nq * LP;
@@ -191,8 +215,10 @@ __global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws) {
     __syncthreads();
   }
   int run_p = s_pts[threadIdx.x] - pts, run_c = s_chk[threadIdx.x] - chk;
+  const int per_class = ws.plan->bins_per_class;
   for (int i = lo; i < hi; ++i) {
     const int c = ws.counts[i];
+    if (i % per_class == 0) ws.plan->class_start[i / per_class] = run_c;
     ws.cursor[i] = run_p;
     run_p += c;
     const int k = (c + ch - 1) / ch;
@@ -200,7 +226,10 @@ __global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws) {
     run_c += k;
     ws.chunk_end[i] = run_c;
   }
-  if (threadIdx.x == 1023) ws.plan->total_chunks = s_chk[1023];
+  if (threadIdx.x == 1023) {
+    ws.plan->total_chunks = s_chk[1023];
+    ws.plan->class_start[kClasses] = s_chk[1023];
+  }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -227,7 +256,7 @@ __global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws) {
 #ifdef DFA3D_TILE_TIMING
 #define TT_DECL unsigned long long tt_acc[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long tt_last = clock64();
 #define TT_MARK(i) do { if (threadIdx.x == 0) { const unsigned long long tt_now = clock64(); tt_acc[i] += tt_now - tt_last; tt_last = tt_now; } } while (0)
-#define TT_FLUSH() do { if (threadIdx.x == 0) { unsigned long long *tt_g = reinterpret_cast<unsigned long long *>(ws.queues + 16); for (int i = 0; i < 10; ++i) atomicAdd(tt_g + i, tt_acc[i]); } } while (0)
+#define TT_FLUSH() do { if (threadIdx.x == 0) { unsigned long long *tt_g = reinterpret_cast<unsigned long long *>(ws.queues + kClasses * kQueueStride); for (int i = 0; i < 10; ++i) atomicAdd(tt_g + i, tt_acc[i]); } } while (0)
 #else
 #define TT_DECL
 #define TT_MARK(i) do { } while (0)
@@ -250,6 +279,21 @@ __host__ __device__ inline TileLds tile_lds_layout(int ty, int tx, int C, int D,
   o.goff = o.offs + R + 1;
   o.total = o.goff + PP;
   return o;
+}
+
+// Thread 0 of a tile workgroup: next work item, from the queue of the workgroup's own class first and
+// from the other classes once that is empty; -1 when every queue is drained.
+__device__ __forceinline__ int pop_item(const BinWorkspace &ws, const BinPlan &p, int home, int &classes_done) {
+  while (classes_done < kClasses) {
+    const int c = (home + classes_done) % kClasses;
+    const int lo = p.class_start[c], hi = p.class_start[c + 1];
+    if (lo < hi) {
+      const int w = lo + atomicAdd(&ws.queues[c * kQueueStride], 1);
+      if (w < hi) return w;
+    }
+    ++classes_done;
+  }
+  return -1;
 }
 
 struct RowTask { float w; uint32_t who; };   // who = point slot * 4 + corner: the index of the task's dot
@@ -336,14 +380,14 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
   for (int i = tid; i < R * (C + D); i += n_thr) smem[i] = 0;   // gv and gd are adjacent
   TT_DECL
 
-  const int total_chunks = p.total_chunks, CH = p.chunk;
+  const int CH = p.chunk;
+  int classes_done = 0;                                   // thread 0: queues found empty so far
   for (;;) {
     // ---- next work item: (bin, chunk of its points), in bin order
     __syncthreads();
     if (tid == 0) {
-      const int w = atomicAdd(&ws.queues[0], 1);
-      const int bin = w < total_chunks ? ws.item_bin[w] : -1;
-      s_bin = bin;
+      const int w = pop_item(ws, p, blockIdx.x % kClasses, classes_done);
+      s_bin = w >= 0 ? ws.item_bin[w] : -1;
       s_item = w;
     }
     __syncthreads();
@@ -357,7 +401,8 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
     const int n_item = min(CH, n_bin - first);
     const int seg = ws.cursor[bin] - n_bin + first;       // the fill advanced the cursor to the segment's end
     const int bm = bin / nb, local = bin - bm * nb;
-    const int b = bm / M, m = bm - b * M;
+    int b, m;
+    slot_decode(bm, B, M, b, m);
     int l = 0;
     while (l + 1 < L && local >= p.level_base[l + 1]) ++l;
     const int tile = local - p.level_base[l];
@@ -684,12 +729,13 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
   const int tid = threadIdx.x, n_thr = blockDim.x;
   float *gd = smem;
   for (int i = tid; i < R * D; i += n_thr) gd[i] = 0;
-  const int total_chunks = p.total_chunks, CH = p.chunk;
+  const int CH = p.chunk;
+  int classes_done = 0;                                   // thread 0: queues found empty so far
   for (;;) {
     __syncthreads();
     if (tid == 0) {
-      const int w = atomicAdd(&ws.queues[0], 1);
-      s_bin = w < total_chunks ? ws.item_bin[w] : -1;
+      const int w = pop_item(ws, p, blockIdx.x % kClasses, classes_done);
+      s_bin = w >= 0 ? ws.item_bin[w] : -1;
       s_item = w;
     }
     __syncthreads();
@@ -702,7 +748,8 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
     const int n_item = min(CH, n_bin - first);
     const int seg = ws.cursor[bin] - n_bin + first;
     const int bm = bin / nb, local = bin - bm * nb;
-    const int b = bm / M, m = bm - b * M;
+    int b, m;
+    slot_decode(bm, B, M, b, m);
     int l = 0;
     while (l + 1 < L && local >= p.level_base[l + 1]) ++l;
     const int tile = local - p.level_base[l];
@@ -764,12 +811,12 @@ constexpr int kMinChunk = 64;        // smallest accepted points-per-item
 struct BinLayout { size_t plan, queues, counts, cursor, chunk_end, item_bin, entries, recs, total; };
 static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
   BinLayout o;
-  const size_t nbins = (size_t)max_bins_per_bm(a.S, a.L, ty, tx) * a.B * a.M;
+  const size_t nbins = (size_t)max_bins_per_bm(a.S, a.L, ty, tx) * slot_count(a.B, a.M);
   const size_t npts = (size_t)a.B * a.Q * a.M * a.L * a.P;
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
   o.plan = 0;
   o.queues = up(o.plan + sizeof(BinPlan));
-  o.counts = up(o.queues + kQueues * sizeof(int));
+  o.counts = up(o.queues + kQueueInts * sizeof(int));
   o.cursor = up(o.counts + nbins * sizeof(int));
   o.chunk_end = up(o.cursor + nbins * sizeof(int));
   // work items: at most one partial chunk per bin plus the full chunks
