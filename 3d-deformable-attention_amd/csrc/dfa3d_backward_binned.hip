@@ -29,7 +29,7 @@ namespace dfa3d {
 constexpr int kClasses = 8;         // work queues: one per XCD (workgroup id % 8 with round-robin placement)
 constexpr int kQueueStride = 16;    // ints between queue counters: one 64-byte line each
 constexpr int kQueueInts = kClasses * kQueueStride + 32;   // + room for the optional phase timers
-constexpr int kBinQueries = 64;     // queries of one (batch, head) handled by a count/fill block
+constexpr int kBinQueries = 32;     // queries of one (batch, head) handled by a count/fill block (16, 64, 128 time worse)
 constexpr int kHistCap = 8192;      // bins of one (batch, head) that fit the LDS histogram
 
 struct BinPlan {
