@@ -92,7 +92,7 @@ int dfa3d_stream_copy(void *dst, const void *src, size_t bytes, void *stream) {
 }
 
 const char *dfa3d_last_error(void) { return g_err; }
-int dfa3d_abi_version(void) { return 4; }
+int dfa3d_abi_version(void) { return 5; }
 
 int dfa3d_set_tunable(const char *name, int value) {
   if (name == nullptr) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: name is NULL");
@@ -321,6 +321,34 @@ int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *sha
     if (e != hipErrorNotSupported) return hip_result(e, fn);
   }
   return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
+}
+
+static int check_rebatch(const char *fn, int bs, int cams, int max_len, int Nq, int E, int dtype) {
+  if (dtype != DFA3D_F32 && dtype != DFA3D_F64) return fail(DFA3D_EINVAL, "%s: dtype must be DFA3D_F32 or DFA3D_F64", fn);
+  if (bs <= 0 || cams <= 0 || max_len <= 0 || Nq <= 0 || E <= 0)
+    return fail(DFA3D_EINVAL, "%s: dimensions must be positive (bs=%d cams=%d max_len=%d Nq=%d E=%d)", fn, bs, cams,
+                max_len, Nq, E);
+  return 0;
+}
+
+int dfa3d_rebatch_gather(const void *src, long long cam_stride, long long batch_stride, const int32_t *index,
+                         const void *scale, void *dst, int bs, int cams, int max_len, int Nq, int E, int dtype,
+                         void *stream) {
+  const char *fn = "dfa3d_rebatch_gather";
+  if (int rc = check_rebatch(fn, bs, cams, max_len, Nq, E, dtype)) return rc;
+  if (cam_stride < 0 || batch_stride < 0) return fail(DFA3D_EINVAL, "%s: strides must not be negative", fn);
+  REQUIRE_PTR(fn, src); REQUIRE_PTR(fn, index); REQUIRE_PTR(fn, dst);
+  return hip_result(dfa3d::launch_rebatch_gather(src, cam_stride, batch_stride, index, scale, dst, bs, cams, max_len,
+                                                 Nq, E, dtype, (hipStream_t)stream), fn);
+}
+
+int dfa3d_rebatch_combine(const void *src, const int32_t *pos, const void *scale, void *dst, int bs, int cams,
+                          int max_len, int Nq, int E, int dtype, void *stream) {
+  const char *fn = "dfa3d_rebatch_combine";
+  if (int rc = check_rebatch(fn, bs, cams, max_len, Nq, E, dtype)) return rc;
+  REQUIRE_PTR(fn, src); REQUIRE_PTR(fn, pos); REQUIRE_PTR(fn, dst);
+  return hip_result(dfa3d::launch_rebatch_combine(src, pos, scale, dst, bs, cams, max_len, Nq, E, dtype,
+                                                  (hipStream_t)stream), fn);
 }
 
 }  // extern "C"

@@ -95,4 +95,11 @@ size_t binned_depth_score_backward_workspace_bytes(const DepthScoreBwdArgs &d, i
 hipError_t launch_depth_score_backward_binned(const DepthScoreBwdArgs &d, int dtype, void *workspace,
                                               size_t workspace_bytes, int tile_hint, int chunk_hint, hipStream_t stream);
 
+// Camera re-batching (dfa3d_rebatch.hip); strides in elements.
+hipError_t launch_rebatch_gather(const void *src, long long cam_stride, long long batch_stride, const int *index,
+                                 const void *scale, void *dst, int bs, int cams, int max_len, int Nq, int E,
+                                 int dtype, hipStream_t stream);
+hipError_t launch_rebatch_combine(const void *src, const int *pos, const void *scale, void *dst, int bs, int cams,
+                                  int max_len, int Nq, int E, int dtype, hipStream_t stream);
+
 }  // namespace dfa3d

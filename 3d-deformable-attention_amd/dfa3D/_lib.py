@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdfa3d_hip.so")
 
 DFA3D_F32, DFA3D_F64, DFA3D_BF16 = 0, 1, 2
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _P, _I = ctypes.c_void_p, ctypes.c_int
 _DIMS7 = [_I] * 7      # B S M (C|D) L Q P
@@ -27,6 +27,8 @@ SIGNATURES = {
     + _DIMS7 + [_I, _P],
     "dfa3d_fused_forward": [_P] * 9 + _DIMS8 + [_I, _I, _P],
     "dfa3d_fused_backward": [_P] * 14 + [ctypes.c_size_t] + _DIMS8 + [_I, _I, _P],
+    "dfa3d_rebatch_gather": [_P, ctypes.c_longlong, ctypes.c_longlong, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "dfa3d_rebatch_combine": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "dfa3d_set_tunable": [ctypes.c_char_p, _I],
     "dfa3d_stream_copy": [_P, _P, ctypes.c_size_t, _P],
     "dfa3d_abi_version": [],

@@ -99,6 +99,24 @@ def variant_timings(_ext, torch, value, dist, shapes, lsi, loc, attn, go, reps):
     out["plain_msda_fwd_ms"] = round(event_time(lambda: _ext.ms_deform_attn_forward(value, shapes, lsi, loc, attn, 64),
                                                 reps)[0], 4)
     out["plain_msda_bwd_ms"] = round(event_time(plain_bwd, reps)[0], 4)
+    del gv, gd, gd1, gl, ga
+
+    # camera re-batching at BEVFormer-base size: 200x200 BEV queries of 256 channels, 6 cameras that each see
+    # a random quarter of them (10 000 per camera: the query count of the operator workload above)
+    from dfa3D.rebatch import camera_index, rebatch_combine, rebatch_gather
+    g = torch.Generator().manual_seed(0)
+    hit = (torch.rand(6, 40000, generator=g) < 0.25).to(dev)
+    index, pos, max_len = camera_index(hit)
+    bev = torch.randn(1, 40000, 256, generator=g).to(dev)
+    scale = (1.0 / hit.sum(0).clamp(min=1).float())[None].contiguous()
+    parts = rebatch_gather(bev, index)
+    ms_g = event_time(lambda: rebatch_gather(bev, index), reps)[0]
+    ms_c = event_time(lambda: rebatch_combine(parts, pos, scale), reps)[0]
+    moved = int(hit.sum().item()) * 256 * 4
+    out["rebatch_gather_ms"] = round(ms_g, 4)
+    out["rebatch_gather_gbs"] = round((moved + parts.numel() * 4) / (ms_g * 1e-3) / 1e9, 1)       # rows read + batch written
+    out["rebatch_combine_ms"] = round(ms_c, 4)
+    out["rebatch_combine_gbs"] = round((moved + bev.numel() * 4) / (ms_c * 1e-3) / 1e9, 1)        # rows read + slots written
     return out
 
 

@@ -141,6 +141,25 @@ int dfa3d_fused_backward(
  * apply (DFA3D_F64, rows too long for LDS tiles, more than 2^31 points, invalid dimensions). */
 size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, int L, int Q, int P, int dtype);
 
+/* Camera re-batching around the operator, as DFA3D-BEVFormer's spatial cross-attention does it in python
+ * loops over batch x cameras
+ * (BEVFormer_DFA3D/projects/mmdet3d_plugin/bevformer/modules/spatial_cross_attention.py:716-722, 741-748).
+ * `index` (cams, max_len) int32 lists the BEV queries that project into each camera, padded with -1;
+ * `pos` (cams, Nq) int32 is its inverse: the position of query q in camera i's list, or -1.  Rows have E
+ * contiguous elements; DFA3D_F32 or DFA3D_F64.
+ *
+ * gather:  dst[j,i,k,:] = scale[j,q] * src[i*cam_stride + j*batch_stride + q*E + :], q = index[i,k]; zeros for
+ *          padding.  dst is (bs, cams, max_len, E); strides are in elements (cam_stride 0: one source for all
+ *          cameras); scale (bs, Nq) may be NULL.  Replaces :716-722; also the backward of the combine.
+ * combine: dst[j,q,:] = scale[j,q] * sum over cameras i with pos[i,q] >= 0 of src[j,i,pos[i,q],:], cameras in
+ *          order, no atomics.  src is (bs, cams, max_len, E), dst (bs, Nq, E), every element written; with
+ *          scale = 1 / max(number of cameras seeing q, 1) this replaces :741-748; also the backward of the gather. */
+int dfa3d_rebatch_gather(const void *src, long long cam_stride, long long batch_stride, const int32_t *index,
+                         const void *scale, void *dst, int bs, int cams, int max_len, int Nq, int E, int dtype,
+                         void *stream);
+int dfa3d_rebatch_combine(const void *src, const int32_t *pos, const void *scale, void *dst, int bs, int cams,
+                          int max_len, int Nq, int E, int dtype, void *stream);
+
 /* Message for the last non-zero return on the calling thread ("" if none). */
 const char *dfa3d_last_error(void);
 
