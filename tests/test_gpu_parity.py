@@ -405,6 +405,70 @@ def test_bf16_storage(oracle):
     torch.testing.assert_close(ga.cpu(), o_ga, **F32_BWD)
 
 
+def test_bf16_other_entry_points(oracle):
+    """bfloat16 storage through the two separate stages, through the shared-distribution / weight_update
+    Function and through plain deformable attention, same bounds as test_bf16_storage."""
+    from dfa3D.functional import MultiScale3DDeformableAttnWeightUpdateFunction, MultiScaleDeformableAttnFunction
+    from dfa3D.workloads import WORKLOADS, make_inputs, scaled
+    dev = _dev()
+    w = scaled(WORKLOADS["base_peaky"], B=2, Q=700)
+    inp = make_inputs(w, seed=6)
+    bf = dict(rtol=8e-3, atol=8e-3)
+    r16 = dict(inp, value=inp["value"].bfloat16().float(), value_dpt_dist=inp["value_dpt_dist"].bfloat16().float(),
+               grad_output=inp["grad_output"].bfloat16().float())
+    shapes3, lsi = inp["spatial_shapes"].to(dev), inp["level_start_index"].to(dev)
+
+    def leaves(dist):
+        return [inp["value"].bfloat16().to(dev).requires_grad_(), dist.bfloat16().to(dev).requires_grad_(),
+                inp["sampling_locations"].to(dev).requires_grad_(), inp["attention_weights"].to(dev).requires_grad_()]
+
+    def close_grads(grads, want, gd_scale):
+        torch.testing.assert_close(grads[0].float().cpu(), want[0], **bf)
+        torch.testing.assert_close(grads[1].float().cpu(), want[1], rtol=8e-3, atol=8e-3 * max(1.0, gd_scale))
+        # grad_loc / grad_attn are float32 but see the bf16 rounding of the score tensor in the two-stage form
+        torch.testing.assert_close(grads[2].cpu(), want[2], rtol=2e-2, atol=2e-2 * max(1.0, want[2].abs().max().item()))
+        torch.testing.assert_close(grads[3].cpu(), want[3], rtol=2e-2, atol=2e-2)
+
+    # two stages, score tensor stored in bf16 between them
+    _, F3, F2 = _functions()
+    o_out, o_score, o_gv, o_gd, o_gl, o_ga = _oracle_one_stage(oracle, r16)
+    v, d, loc, a = leaves(inp["value_dpt_dist"])
+    score = F3.apply(d, shapes3, lsi, loc, 64)
+    out = F2.apply(v, shapes3, lsi, loc, a, score, 64)
+    assert score.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+    grads = torch.autograd.grad(out, [v, d, loc, a], inp["grad_output"].bfloat16().to(dev))
+    torch.testing.assert_close(out.float().cpu(), o_out, rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(score.float().cpu(), o_score, **bf)
+    close_grads(grads, (o_gv, o_gd, o_gl, o_ga), o_gd.abs().max().item())
+
+    # one distribution for all heads, weight_update instead of scores
+    shared = dict(r16, value_dpt_dist=r16["value_dpt_dist"][:, :, :1].contiguous())
+    want = _shared_dist_expectation(oracle, shared)
+    v, d, loc, a = leaves(inp["value_dpt_dist"][:, :, :1].contiguous())
+    out, wu = MultiScale3DDeformableAttnWeightUpdateFunction.apply(v, d, shapes3, lsi, loc, a, 64)
+    grads = torch.autograd.grad(out, [v, d, loc, a], inp["grad_output"].bfloat16().to(dev))
+    torch.testing.assert_close(out.float().cpu(), want[0], **bf)
+    torch.testing.assert_close(wu.cpu(), want[2], **F32_FWD)
+    torch.testing.assert_close(grads[0].float().cpu(), want[3], **bf)
+    torch.testing.assert_close(grads[1].float().cpu(), want[4], rtol=8e-3, atol=8e-3 * max(1.0, want[4].abs().max().item()))
+    torch.testing.assert_close(grads[2].cpu(), want[5], **F32_BWD)
+    torch.testing.assert_close(grads[3].cpu(), want[6], **F32_BWD)
+
+    # plain deformable attention
+    ones = torch.ones(*inp["attention_weights"].shape, 4)
+    args = (r16["value"], inp["spatial_shapes"][:, :2].contiguous(), inp["level_start_index"],
+            inp["sampling_locations"][..., :2].contiguous(), inp["attention_weights"], ones)
+    p_out = oracle.wms_forward(*args)
+    p_gv, p_gl, p_ga, _ = oracle.wms_backward(*args, r16["grad_output"])
+    v, _, loc, a = leaves(inp["value_dpt_dist"])
+    out = MultiScaleDeformableAttnFunction.apply(v, shapes3, lsi, loc, a, 64)
+    gv, gl, ga = torch.autograd.grad(out, [v, loc, a], inp["grad_output"].bfloat16().to(dev))
+    torch.testing.assert_close(out.float().cpu(), p_out, rtol=8e-3, atol=8e-3 * max(1.0, p_out.abs().max().item()))
+    torch.testing.assert_close(gv.float().cpu(), p_gv, **bf)
+    torch.testing.assert_close(gl[..., :2].cpu(), p_gl, **F32_BWD)
+    torch.testing.assert_close(ga.cpu(), p_ga, **F32_BWD)
+
+
 def test_nan_in_unsampled_pixel_does_not_leak(oracle):
     """Corners outside the map are never read and never multiplied in."""
     dev = _dev()
