@@ -102,8 +102,8 @@ int dfa3d_set_tunable(const char *name, int value) {
     return 0;
   }
   if (!strcmp(name, "vec")) {
-    if (value != 0 && value != 1 && value != 2 && value != 4)
-      return fail(DFA3D_EINVAL, "dfa3d_set_tunable: vec must be 0 (automatic), 1, 2 or 4");
+    if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8)
+      return fail(DFA3D_EINVAL, "dfa3d_set_tunable: vec must be 0 (automatic), 1, 2, 4 or 8");
     g_vec.store(value, std::memory_order_relaxed);
     return 0;
   }

@@ -344,6 +344,16 @@ template <> struct LdsVec<4> {
     *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
   }
 };
+template <> struct LdsVec<8> {
+  static __device__ __forceinline__ void ld(const float *p, float (&v)[8]) {
+    const float4 t0 = reinterpret_cast<const float4 *>(p)[0], t1 = reinterpret_cast<const float4 *>(p)[1];
+    v[0] = t0.x; v[1] = t0.y; v[2] = t0.z; v[3] = t0.w; v[4] = t1.x; v[5] = t1.y; v[6] = t1.z; v[7] = t1.w;
+  }
+  static __device__ __forceinline__ void st(float *p, const float (&v)[8]) {
+    reinterpret_cast<float4 *>(p)[0] = make_float4(v[0], v[1], v[2], v[3]);
+    reinterpret_cast<float4 *>(p)[1] = make_float4(v[4], v[5], v[6], v[7]);
+  }
+};
 template <int VEC> __device__ __forceinline__ void lds_ld(const float *p, float (&v)[VEC]) { LdsVec<VEC>::ld(p, v); }
 
 // FUSED: both stages (depth scores recomputed from dist, grad_dist and the z gradient produced).
@@ -539,7 +549,9 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
             RowVec<T, float, VEC>::ld(value_r, (ld_ok ? (uint32_t)(((start + yn * W + xn) * M + m) * C * (int)sizeof(T)) : kNoRow) + chan_off, v_next);
           }
           if (n_max == 0) continue;                      // wave-uniform
-          constexpr int UT = 4;
+          // tasks in flight per group: registers decide (measured: 4 with four channels per lane, 1 with eight;
+          // one more costs 1 % .. 10 % of the kernel's time)
+          constexpr int UT = VEC >= 8 ? 1 : 4;
           const RowTask *row_tasks = tasks + beg;
           const int last_task = PP * 4 - 1 - beg;         // reads past a short list stay inside the array
           const float *g_lane = gstage + (chan_ok ? chan : 0);
@@ -917,6 +929,14 @@ static hipError_t launch_tile_cfg(const BwdArgs &a, const BinWorkspace &ws, cons
 
 template <typename T>
 static hipError_t launch_tile_typed(const BwdArgs &a, const BinWorkspace &ws, const TileConfig &c, hipStream_t stream) {
+  // Eight channels per lane when the tile has more rows than four-channel row groups (a 9x9 tile against 64
+  // groups of 8 lanes): 128 groups of 4 lanes then cover it in one round with fewer instructions per corner
+  // task.  Smaller tiles would leave most of those groups idle.
+  const int groups4 = (c.block / 64) * 8;
+  if (((a.vec_hint == 0 && (c.ty + 1) * (c.tx + 1) > groups4) || a.vec_hint == 8) && sizeof(T) <= 4) {
+    if (a.C == 32) return launch_tile_cfg<T, 8, 4>(a, ws, c, stream);
+    if (a.C == 64) return launch_tile_cfg<T, 8, 8>(a, ws, c, stream);
+  }
   const RowTiling rt = pick_row_tiling(a.C, (int)sizeof(T), a.vec_hint);
 #define DFA3D_CASE(V, R) \
   if (rt.vec == V && rt.lpr == R) return launch_tile_cfg<T, V, R>(a, ws, c, stream);

@@ -115,6 +115,14 @@ template <typename A> struct RowVec<float, A, 4> {
     *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
   }
 };
+template <typename A> struct RowVec<float, A, 8> {      // loads only: used by the tile kernels
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[8]) {
+    const u32x4 t0 = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    const u32x4 t1 = __builtin_amdgcn_raw_buffer_load_b128(r, off + 16, 0, 0);
+    v[0] = __uint_as_float(t0.x); v[1] = __uint_as_float(t0.y); v[2] = __uint_as_float(t0.z); v[3] = __uint_as_float(t0.w);
+    v[4] = __uint_as_float(t1.x); v[5] = __uint_as_float(t1.y); v[6] = __uint_as_float(t1.z); v[7] = __uint_as_float(t1.w);
+  }
+};
 template <typename A> struct RowVec<double, A, 1> {
   static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[1]) { v[0] = BufElem<double>::ld(r, off); }
   static __device__ __forceinline__ void st(double *p, const A (&v)[1]) { p[0] = v[0]; }
@@ -168,6 +176,16 @@ template <typename A> struct RowVec<__hip_bfloat16, A, 4> {
   static __device__ __forceinline__ void st(__hip_bfloat16 *p, const A (&v)[4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) p[i] = __float2bfloat16(v[i]);
+  }
+};
+
+template <typename A> struct RowVec<__hip_bfloat16, A, 8> {      // loads only: used by the tile kernels
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, A (&v)[8]) {
+    const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xFFFF0000u);
+    v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xFFFF0000u);
+    v[4] = __uint_as_float(t.z << 16); v[5] = __uint_as_float(t.z & 0xFFFF0000u);
+    v[6] = __uint_as_float(t.w << 16); v[7] = __uint_as_float(t.w & 0xFFFF0000u);
   }
 };
 

@@ -165,7 +165,7 @@ const char *dfa3d_last_error(void);
 
 /* Process-wide launch tunables; results do not depend on them.
  *   "iters"  groups of units each wavefront walks through (default 1)
- *   "vec"    channels per lane in the row gathers: 0 = automatic, 1, 2 or 4
+ *   "vec"    channels per lane in the row gathers: 0 = automatic, 1, 2 or 4 (8: tile kernels only)
  *   "diag"   measurement aid for the backward kernels: bit 0 drops the grad_value updates,
  *            bit 1 the grad_dist updates (results are then incomplete); default 0
  *   "binned" 0 makes dfa3d_fused_backward ignore its workspace (direct atomic kernel); default 1
