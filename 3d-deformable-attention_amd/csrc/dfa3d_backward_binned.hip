@@ -143,13 +143,22 @@ __global__ __launch_bounds__(256) void bin_points_kernel(
     for (int i = threadIdx.x; i < nb * (MODE == 1 ? 2 : 1); i += blockDim.x) s_hist[i] = 0;
     __syncthreads();
   }
-  // pass 1: histogram of this block's points
-  for (int i = threadIdx.x; i < npts; i += blockDim.x) {
+  // pass 1: histogram of this block's points; the fill keeps the bins of its first kKept rounds in registers
+  constexpr int kKept = 4;
+  int kept[kKept];
+#pragma unroll
+  for (int k = 0; k < kKept; ++k) kept[k] = -1;
+  int round = 0;
+  for (int i = threadIdx.x; i < npts; i += blockDim.x, ++round) {
     const int qi = i / LP, lp = i - qi * LP, l = lp / P;
     const size_t gp = ((size_t)(b * (size_t)Q + q0 + qi) * M + m) * LP + lp;
     const Point2D<float> g = locate_2d<float>(loc[gp * loc_stride], loc[gp * loc_stride + 1], p.H[l], p.W[l], p.start[l]);
     if (g.inside && p.tiles_x[l] > 0) {
       const int bin = bin_of(p, l, g);
+      if (MODE == 1) {
+#pragma unroll
+        for (int k = 0; k < kKept; ++k) kept[k] = round == k ? bin : kept[k];
+      }
       if (use_lds) atomicAdd(&s_hist[bin], 1);
       else if (MODE == 0) atomicAdd(&gcount[bin], 1);
     } else if (MODE == 1) {
@@ -175,12 +184,19 @@ __global__ __launch_bounds__(256) void bin_points_kernel(
   }
   if (MODE == 1) {
     // pass 2: place the points
-    for (int i = threadIdx.x; i < npts; i += blockDim.x) {
+    round = 0;
+    for (int i = threadIdx.x; i < npts; i += blockDim.x, ++round) {
       const int qi = i / LP, lp = i - qi * LP, l = lp / P;
       const size_t gp = ((size_t)(b * (size_t)Q + q0 + qi) * M + m) * LP + lp;
-      const Point2D<float> g = locate_2d<float>(loc[gp * loc_stride], loc[gp * loc_stride + 1], p.H[l], p.W[l], p.start[l]);
-      if (g.inside && p.tiles_x[l] > 0) {
-        const int bin = bin_of(p, l, g);
+      int bin = -1;
+      if (round < kKept) {
+#pragma unroll
+        for (int k = 0; k < kKept; ++k) bin = round == k ? kept[k] : bin;
+      } else {
+        const Point2D<float> g = locate_2d<float>(loc[gp * loc_stride], loc[gp * loc_stride + 1], p.H[l], p.W[l], p.start[l]);
+        if (g.inside && p.tiles_x[l] > 0) bin = bin_of(p, l, g);
+      }
+      if (bin >= 0) {
         const int slot = use_lds ? s_hist[nb + bin] + atomicAdd(&s_hist[bin], 1) : atomicAdd(&gcursor[bin], 1);
         if (!(diag & 128)) ws.entries[slot] = (uint32_t)gp;
         if (!(diag & 64))
@@ -192,43 +208,52 @@ __global__ __launch_bounds__(256) void bin_points_kernel(
 }
 
 __global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws) {
-  __shared__ int s_pts[1024], s_chk[1024];
-  const int n = ws.plan->total_bins, ch = ws.plan->chunk;
-  const int per = (n + 1023) / 1024;
-  const int lo = min(n, (int)threadIdx.x * per), hi = min(n, lo + per);
-  int pts = 0, chk = 0;
-  for (int i = lo; i < hi; ++i) {
-    const int c = ws.counts[i];
-    pts += c;
-    chk += (c + ch - 1) / ch;
-  }
-  s_pts[threadIdx.x] = pts;
-  s_chk[threadIdx.x] = chk;
+  // One workgroup walks the bins 4096 at a time: four consecutive bins per thread (their loads are
+  // independent, so a round costs one memory latency), a workgroup-wide exclusive scan of points and of
+  // work items, and a running carry.
+  __shared__ int s_pts[16], s_chk[16], s_carry[2];
+  const int n = ws.plan->total_bins, ch = ws.plan->chunk, per_class = ws.plan->bins_per_class;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  if (threadIdx.x == 0) { s_carry[0] = 0; s_carry[1] = 0; }
   __syncthreads();
-  // inclusive scans of the 1024 partial sums (Hillis-Steele, a barrier pair per step)
-  for (int off = 1; off < 1024; off <<= 1) {
-    const int ap = threadIdx.x >= (unsigned)off ? s_pts[threadIdx.x - off] : 0;
-    const int ac = threadIdx.x >= (unsigned)off ? s_chk[threadIdx.x - off] : 0;
+  for (int base = 0; base < n; base += 4096) {
+    const int i0 = base + (int)threadIdx.x * 4;
+    int c[4], k[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      c[j] = i0 + j < n ? ws.counts[i0 + j] : 0;
+      k[j] = (c[j] + ch - 1) / ch;
+    }
+    const int pts = c[0] + c[1] + c[2] + c[3], chk = k[0] + k[1] + k[2] + k[3];
+    int ip = pts, ic = chk;                                  // inclusive scans within the wavefront
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const int up = __shfl_up(ip, off, kWave), uc = __shfl_up(ic, off, kWave);
+      if (lane >= off) { ip += up; ic += uc; }
+    }
+    if (lane == kWave - 1) { s_pts[wave] = ip; s_chk[wave] = ic; }
     __syncthreads();
-    s_pts[threadIdx.x] += ap;
-    s_chk[threadIdx.x] += ac;
+    int run_p = s_carry[0] + ip - pts, run_c = s_carry[1] + ic - chk;
+    for (int w = 0; w < wave; ++w) { run_p += s_pts[w]; run_c += s_chk[w]; }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = i0 + j;
+      if (i < n) {
+        if (i % per_class == 0) ws.plan->class_start[i / per_class] = run_c;
+        ws.cursor[i] = run_p;
+        run_p += c[j];
+        for (int t = 0; t < k[j]; ++t) ws.item_bin[run_c + t] = i;
+        run_c += k[j];
+        ws.chunk_end[i] = run_c;
+      }
+    }
+    __syncthreads();                                         // everyone has read the carry and the wave sums
+    if (threadIdx.x == 1023) { s_carry[0] = run_p; s_carry[1] = run_c; }
     __syncthreads();
   }
-  int run_p = s_pts[threadIdx.x] - pts, run_c = s_chk[threadIdx.x] - chk;
-  const int per_class = ws.plan->bins_per_class;
-  for (int i = lo; i < hi; ++i) {
-    const int c = ws.counts[i];
-    if (i % per_class == 0) ws.plan->class_start[i / per_class] = run_c;
-    ws.cursor[i] = run_p;
-    run_p += c;
-    const int k = (c + ch - 1) / ch;
-    for (int j = 0; j < k; ++j) ws.item_bin[run_c + j] = i;
-    run_c += k;
-    ws.chunk_end[i] = run_c;
-  }
-  if (threadIdx.x == 1023) {
-    ws.plan->total_chunks = s_chk[1023];
-    ws.plan->class_start[kClasses] = s_chk[1023];
+  if (threadIdx.x == 0) {
+    ws.plan->total_chunks = s_carry[1];
+    ws.plan->class_start[kClasses] = s_carry[1];
   }
 }
 
