@@ -88,7 +88,14 @@ def test_fp64_one_stage_matches_checker(oracle, case):
     _compare(got, want, dict(rtol=1e-10, atol=1e-11), dict(rtol=1e-10, atol=1e-11))
 
 
-@pytest.mark.parametrize("case", TINY[:4], ids=lambda c: f"seed{c['seed']}")
+FP32_EXTRA = [
+    dict(seed=8, C=48, M=12, Q=11, P=3, D=10, levels=((9, 7), (5, 4), (2, 3))),   # 12 heads: two heads per XCD class
+    dict(seed=9, C=64, M=16, Q=40, P=4, D=6, levels=((20, 31), (10, 16))),        # C=64: eight channels per lane
+    dict(seed=10, C=32, M=5, Q=300, P=8, D=64, levels=((33, 47), (17, 24), (9, 12), (5, 6))),   # several tiles per level
+]
+
+
+@pytest.mark.parametrize("case", TINY + FP32_EXTRA, ids=lambda c: f"seed{c['seed']}")
 def test_fp32_one_stage_matches_checker_tiny(oracle, case):
     dev = _dev()
     t = tiny_case(**case)
