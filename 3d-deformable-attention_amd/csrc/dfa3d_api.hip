@@ -92,7 +92,7 @@ int dfa3d_stream_copy(void *dst, const void *src, size_t bytes, void *stream) {
 }
 
 const char *dfa3d_last_error(void) { return g_err; }
-int dfa3d_abi_version(void) { return 5; }
+int dfa3d_abi_version(void) { return 6; }
 
 int dfa3d_set_tunable(const char *name, int value) {
   if (name == nullptr) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: name is NULL");
@@ -292,12 +292,14 @@ static dfa3d::BwdArgs fused_bwd_args(const void *value, const void *dist, const 
   return a;
 }
 
-size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, int L, int Q, int P, int dtype) {
+size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads,
+                                            int dtype) {
   if (check_dims("dfa3d_fused_backward_workspace_bytes", B, S, M, C, L, Q, P, dtype)) return 0;
   if (check_dims("dfa3d_fused_backward_workspace_bytes", B, S, M, D, L, Q, P, dtype)) return 0;
   if (!g_binned.load(std::memory_order_relaxed)) return 0;
   const dfa3d::BwdArgs a = fused_bwd_args(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
-                                          nullptr, nullptr, nullptr, nullptr, nullptr, B, S, M, C, D, L, Q, P, M);
+                                          nullptr, nullptr, nullptr, nullptr, nullptr, B, S, M, C, D, L, Q, P,
+                                          dist_heads == 1 ? 1 : M);
   return dfa3d::binned_backward_workspace_bytes(a, 0, dtype);
 }
 

@@ -390,7 +390,8 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
     const T *__restrict__ grad_out, const T *__restrict__ grad_score_in,
     float *__restrict__ grad_value, float *__restrict__ grad_dist, float *__restrict__ grad_loc, int gl_stride,
     float *__restrict__ grad_attn, float *__restrict__ grad_score_out, const float *__restrict__ grad_wu, int Md,
-    int B, int S, int M, int C, int D, int L, int Q, int P, int PP, int diag) {
+    int Mg, int B, int S, int M, int C, int D, int L, int Q, int P, int PP, int diag) {
+  // Md: heads stored in dist (M, or 1 = shared by all heads); Mg: heads of the grad_dist buffer written here
   constexpr int RPI = kWave / LPR;                  // row groups per wavefront
   extern __shared__ __align__(16) float smem[];
   __shared__ int s_bin, s_item;
@@ -672,14 +673,15 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
 
     // ---------------- flush the tile (and leave it zeroed for the next item) ----------------
     float *gvalue_b = grad_value + (size_t)b * S * M * C;
-    float *gdist_b = FUSED ? grad_dist + (size_t)b * S * Md * D : nullptr;
+    const int mg = Mg == 1 ? 0 : m;
+    float *gdist_b = FUSED ? grad_dist + (size_t)b * S * Mg * D : nullptr;
     const rsrc_t gvalue_r = make_rsrc(gvalue_b, (size_t)S * M * C * sizeof(float));
-    const rsrc_t gdist_r = make_rsrc(gdist_b, FUSED ? (size_t)S * Md * D * sizeof(float) : 0);
+    const rsrc_t gdist_r = make_rsrc(gdist_b, FUSED ? (size_t)S * Mg * D * sizeof(float) : 0);
     // Rows 1..TY-1 x 1..TX-1 of the tile belong to no neighbour's halo; when this item holds all the
     // points of its bin nobody else adds to them, so they are stored instead of added atomically
     // (grad_value and grad_dist are zero on entry).
     const bool sole = chunks_here == 1;
-    const bool sole_d = sole && Md == M;                 // a distribution shared by the heads collects from all of them
+    const bool sole_d = sole && Mg == M;                 // a gradient shared by the heads collects from all of them
     if (((C | D) & 3) == 0) {
       // four floats per lane: whole 128-byte lines leave each row group at once
       const int c4n = C >> 2, d4n = D >> 2;
@@ -710,7 +712,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const int ry = r / TW, rx = r - ry * TW;
         const int y = y0 + ry, x = x0 + rx;
         if (y < H && x < W && !(diag & 4)) {
-          const uint32_t off = (uint32_t)((((start + y * W + x) * Md + md) * D + d) * 4);
+          const uint32_t off = (uint32_t)((((start + y * W + x) * Mg + mg) * D + d) * 4);
           if (sole_d && ry >= 1 && ry < TY && rx >= 1 && rx < TX) {
             *reinterpret_cast<float4 *>(gdist_b + (off >> 2)) = val;
           } else if (nz) {
@@ -739,7 +741,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const int r = i / D, d = i - r * D;
         const int ry = r / TW, rx = r % TW;
         const int y = y0 + ry, x = x0 + rx;
-        if (y < H && x < W && !(diag & 4)) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * Md + md) * D + d) * 4), val);
+        if (y < H && x < W && !(diag & 4)) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * Mg + mg) * D + d) * 4), val);
       }
     }
     }
@@ -845,7 +847,42 @@ static int max_bins_per_bm(int S, int L, int ty, int tx) {
 }
 
 constexpr int kMinChunk = 64;        // smallest accepted points-per-item
-struct BinLayout { size_t plan, queues, counts, cursor, chunk_end, item_bin, entries, recs, total; };
+// only the fused entry point sets dist_heads
+static bool shared_dist(const BwdArgs &a) { return a.dist_heads == 1 && a.M > 1; }
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(float4 *__restrict__ dst, size_t n4) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256)
+    dst[i] = make_float4(0, 0, 0, 0);
+}
+
+// dst[r, :] = sum over heads m of src[r, m, :], rows of D floats, heads in order
+__global__ __launch_bounds__(256) void head_sum_kernel(const float *__restrict__ src, float *__restrict__ dst,
+                                                       size_t rows, int M, int D) {
+  if ((D & 3) == 0) {
+    const int d4 = D >> 2;
+    const size_t n = rows * d4;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+      const size_t r = i / d4;
+      const int d = (int)(i - r * d4) << 2;
+      float4 acc = make_float4(0, 0, 0, 0);
+      for (int m = 0; m < M; ++m) {
+        const float4 t = *reinterpret_cast<const float4 *>(src + (r * M + m) * D + d);
+        acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+      }
+      *reinterpret_cast<float4 *>(dst + r * D + d) = acc;
+    }
+  } else {
+    const size_t n = rows * D;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+      const size_t r = i / D;
+      const int d = (int)(i - r * D);
+      float acc = 0;
+      for (int m = 0; m < M; ++m) acc += src[(r * M + m) * D + d];
+      dst[i] = acc;
+    }
+  }
+}
+struct BinLayout { size_t plan, queues, counts, cursor, chunk_end, item_bin, entries, recs, gd_heads, total; };
 static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
   BinLayout o;
   const size_t nbins = (size_t)max_bins_per_bm(a.S, a.L, ty, tx) * slot_count(a.B, a.M);
@@ -860,7 +897,11 @@ static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
   o.item_bin = up(o.chunk_end + nbins * sizeof(int));
   o.entries = up(o.item_bin + (nbins + npts / kMinChunk + 1) * sizeof(int));
   o.recs = up(o.entries + npts * sizeof(uint32_t));
-  o.total = up(o.recs + npts * sizeof(float4));
+  // a distribution shared by the heads: grad_dist per head first (stores, as with a distribution per head),
+  // summed over the heads afterwards; eight XCDs adding atomically into one shared tile cost twice as much
+  o.gd_heads = up(o.recs + npts * sizeof(float4));
+  const size_t per_head = shared_dist(a) ? (size_t)a.B * a.S * a.M * a.D * sizeof(float) : 0;
+  o.total = up(o.gd_heads + per_head);
   return o;
 }
 
@@ -930,41 +971,45 @@ template <typename K> static hipError_t allow_lds(K kern, size_t lds) {
 }
 
 template <typename T, int VEC, int LPR>
-static hipError_t launch_tile_cfg(const BwdArgs &a, const BinWorkspace &ws, const TileConfig &c, hipStream_t stream) {
+static hipError_t launch_tile_cfg(const BwdArgs &a, const BinWorkspace &ws, const TileConfig &c, float *gd_heads,
+                                  hipStream_t stream) {
+  // gd_heads != nullptr: the kernel writes grad_dist per head there instead of into a.grad_dist
   const int grid = tile_grid(c.lds, c.block);
   if (a.dist != nullptr) {
     auto kern = tile_backward_kernel<T, VEC, LPR, true>;
     if (hipError_t e = allow_lds(kern, c.lds)) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(c.block), c.lds, stream, ws, (const T *)a.value, (const T *)a.dist,
                        (const T *)nullptr, (const T *)a.grad_out, (const T *)a.grad_score_in, (float *)a.grad_value,
-                       (float *)a.grad_dist, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
-                       (float *)nullptr, (const float *)a.grad_weight_update, a.dist_heads == 1 ? 1 : a.M, a.B, a.S,
-                       a.M, a.C, a.D, a.L, a.Q, a.P, c.pp, a.diag);
+                       gd_heads != nullptr ? gd_heads : (float *)a.grad_dist, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
+                       (float *)nullptr, (const float *)a.grad_weight_update, a.dist_heads == 1 ? 1 : a.M,
+                       (a.dist_heads == 1 && gd_heads == nullptr) ? 1 : a.M, a.B, a.S, a.M, a.C, a.D, a.L, a.Q, a.P, c.pp,
+                       a.diag);
   } else {
     auto kern = tile_backward_kernel<T, VEC, LPR, false>;
     if (hipError_t e = allow_lds(kern, c.lds)) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(c.block), c.lds, stream, ws, (const T *)a.value, (const T *)nullptr,
                        (const T *)a.score_in, (const T *)a.grad_out, (const T *)nullptr, (float *)a.grad_value,
                        (float *)nullptr, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
-                       (float *)a.grad_score_out, (const float *)nullptr, a.M, a.B, a.S, a.M, a.C, 0, a.L, a.Q, a.P,
-                       c.pp, a.diag);
+                       (float *)a.grad_score_out, (const float *)nullptr, a.M, a.M, a.B, a.S, a.M, a.C, 0, a.L, a.Q,
+                       a.P, c.pp, a.diag);
   }
   return hipGetLastError();
 }
 
 template <typename T>
-static hipError_t launch_tile_typed(const BwdArgs &a, const BinWorkspace &ws, const TileConfig &c, hipStream_t stream) {
+static hipError_t launch_tile_typed(const BwdArgs &a, const BinWorkspace &ws, const TileConfig &c, float *gd_heads,
+                                    hipStream_t stream) {
   // Eight channels per lane when the tile has more rows than four-channel row groups (a 9x9 tile against 64
   // groups of 8 lanes): 128 groups of 4 lanes then cover it in one round with fewer instructions per corner
   // task.  Smaller tiles would leave most of those groups idle.
   const int groups4 = (c.block / 64) * 8;
   if (((a.vec_hint == 0 && (c.ty + 1) * (c.tx + 1) > groups4) || a.vec_hint == 8) && sizeof(T) <= 4) {
-    if (a.C == 32) return launch_tile_cfg<T, 8, 4>(a, ws, c, stream);
-    if (a.C == 64) return launch_tile_cfg<T, 8, 8>(a, ws, c, stream);
+    if (a.C == 32) return launch_tile_cfg<T, 8, 4>(a, ws, c, gd_heads, stream);
+    if (a.C == 64) return launch_tile_cfg<T, 8, 8>(a, ws, c, gd_heads, stream);
   }
   const RowTiling rt = pick_row_tiling(a.C, (int)sizeof(T), a.vec_hint);
 #define DFA3D_CASE(V, R) \
-  if (rt.vec == V && rt.lpr == R) return launch_tile_cfg<T, V, R>(a, ws, c, stream);
+  if (rt.vec == V && rt.lpr == R) return launch_tile_cfg<T, V, R>(a, ws, c, gd_heads, stream);
   DFA3D_ROW_TILINGS(DFA3D_CASE)
 #undef DFA3D_CASE
   return hipErrorInvalidValue;
@@ -1016,13 +1061,23 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
   if (need == 0 || workspace == nullptr || workspace_bytes < need || ((uintptr_t)workspace & 255) != 0)
     return hipErrorNotSupported;
   const TileConfig cfg = tile_config_of(a, kind);
-  const BinWorkspace ws = carve_workspace(workspace, bin_layout(a, cfg.ty, cfg.tx));
+  const BinLayout lay = bin_layout(a, cfg.ty, cfg.tx);
+  const BinWorkspace ws = carve_workspace(workspace, lay);
+  float *gd_heads = shared_dist(a) ? reinterpret_cast<float *>(static_cast<char *>(workspace) + lay.gd_heads) : nullptr;
   if (a.stage == 0 || a.stage == 1) {
     if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, stream)) return e;
   }
   if (a.stage == 1) return hipSuccess;
-  if (dtype == DFA3D_F32) return launch_tile_typed<float>(a, ws, cfg, stream);
-  return launch_tile_typed<__hip_bfloat16>(a, ws, cfg, stream);
+  const size_t head_floats = (size_t)a.B * a.S * a.M * a.D;
+  if (gd_heads != nullptr)       // a kernel, not a memset node: callers may capture this stream in a graph
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(2048), dim3(256), 0, stream, reinterpret_cast<float4 *>(gd_heads),
+                       (head_floats + 3) / 4);
+  const hipError_t e = dtype == DFA3D_F32 ? launch_tile_typed<float>(a, ws, cfg, gd_heads, stream)
+                                          : launch_tile_typed<__hip_bfloat16>(a, ws, cfg, gd_heads, stream);
+  if (e != hipSuccess || gd_heads == nullptr) return e;
+  hipLaunchKernelGGL(head_sum_kernel, dim3(2048), dim3(256), 0, stream, gd_heads, (float *)a.grad_dist,
+                     (size_t)a.B * a.S, a.M, a.D);
+  return hipGetLastError();
 }
 
 // Binned backward of stage 1 alone.

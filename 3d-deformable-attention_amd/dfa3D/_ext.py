@@ -360,7 +360,7 @@ def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_leve
         return
     code = _lib.dtype_code(value)
     # scratch for the binned (LDS-accumulating) kernels; 0 bytes means the direct kernel is used
-    ws_bytes = _lib.lib().dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, code)
+    ws_bytes = _lib.lib().dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2], code)
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
     with torch.cuda.device(dev):
         rc = _lib.lib().dfa3d_fused_backward(

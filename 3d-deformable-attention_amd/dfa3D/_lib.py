@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdfa3d_hip.so")
 
 DFA3D_F32, DFA3D_F64, DFA3D_BF16 = 0, 1, 2
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _P, _I = ctypes.c_void_p, ctypes.c_int
 _DIMS7 = [_I] * 7      # B S M (C|D) L Q P
@@ -50,7 +50,7 @@ def lib():
             fn = getattr(handle, name)
             fn.argtypes = argtypes
             fn.restype = ctypes.c_int
-        for name, dims in (("dfa3d_fused_backward_workspace_bytes", _DIMS8),
+        for name, dims in (("dfa3d_fused_backward_workspace_bytes", _DIMS8 + [_I]),
                            ("dfa3d_wms_deform_attn_backward_workspace_bytes", _DIMS7),
                            ("dfa3d_ms_depth_score_sample_backward_workspace_bytes", _DIMS7)):
             fn = getattr(handle, name)

@@ -243,7 +243,7 @@ def main():
     gl = torch.empty_like(loc)
     ga = torch.empty_like(attn)
     vd, dd, ld, ad = value.detach(), dist.detach(), loc.detach(), attn.detach()
-    ws_bytes = L_.dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, code)
+    ws_bytes = L_.dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, dist.shape[2], code)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     stream = _lib.stream_of(value)
 

@@ -138,8 +138,11 @@ int dfa3d_fused_backward(
     int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype, void *stream);
 
 /* Scratch bytes dfa3d_fused_backward wants for these dimensions; 0 when the binned path does not
- * apply (DFA3D_F64, rows too long for LDS tiles, more than 2^31 points, invalid dimensions). */
-size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, int L, int Q, int P, int dtype);
+ * apply (DFA3D_F64, rows too long for LDS tiles, more than 2^31 points, invalid dimensions).  With
+ * dist_heads = 1 this includes B*S*M*D floats: grad_dist is formed per head and summed over the heads
+ * by a last kernel. */
+size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads,
+                                            int dtype);
 
 /* Camera re-batching around the operator, as DFA3D-BEVFormer's spatial cross-attention does it in python
  * loops over batch x cameras
