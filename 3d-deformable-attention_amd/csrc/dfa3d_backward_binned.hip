@@ -3,20 +3,23 @@
 //
 // Why: device-memory atomics retire at roughly 10^10 cache-line requests per second on this part,
 // and the straightforward backward (bwd_attention_kernel) needs 4 row updates of grad_value and 8
-// scalar updates of grad_dist per sampling point.  LDS atomics are two orders of magnitude faster.
-// So the points are first binned by the image tile they fall in, and one workgroup per tile
-// accumulates that tile of grad_value and grad_dist in LDS and writes it out once.
+// scalar updates of grad_dist per sampling point.  So the points are first binned by the image tile they
+// fall in, and one workgroup per tile accumulates that tile of grad_value and grad_dist in LDS and writes it
+// out once: grad_value rows without any atomics (a lane group owns each tile row), grad_dist taps with
+// LDS atomics, which are some 25 times faster than device-memory ones.
 //
-//   plan_and_clear_kernel  validates the level table, lays out the tiles (bins), clears counters
-//   bin_count_kernel       points per bin (LDS histogram per block, one atomic per touched bin)
-//   bin_scan_kernel        exclusive prefix over bins
-//   bin_fill_kernel        writes each point's index into its bin's segment; zero gradients for
-//                          points the operator skips
-//   tile_backward_kernel   persistent workgroups pull (bin, chunk of its points) work items from a
-//                          queue; per item: LDS tiles
-//                          of (TY+1) x (TX+1) pixels (one-pixel halo to the right/bottom, so all four
-//                          corners of a point of this bin land in the tile), the same three phases
-//                          as the direct kernel with LDS atomics, then one flush of the tile
+//   plan_and_clear_kernel       validates the level table, lays out the tiles (bins), clears counters
+//   bin_points_kernel<0>        points per bin (LDS histogram per block, one atomic per touched bin)
+//   bin_scan_kernel             exclusive prefix over bins, work items (bin, chunk of its points)
+//   bin_points_kernel<1>        writes each point's index and record into its bin's segment; zero
+//                               gradients for points the operator skips
+//   tile_backward_kernel        persistent workgroups pull work items from per-XCD queues; per item: LDS
+//                               tiles of (TY+1) x (TX+1) pixels (one-pixel halo to the right/bottom, so
+//                               all four corners of a point of this bin land in the tile), the phases
+//                               described above the kernel, then one flush of the tile.  FUSED=false:
+//                               stage 2 alone
+//   tile_depth_backward_kernel  stage 1 alone on the same bins
+//   fill_zero / head_sum        a distribution shared by the heads: grad_dist per head, then summed
 //
 // A point belongs to the tile that holds its clamped base pixel (clamp(h0,0,H-1), clamp(w0,0,W-1)).
 // Semantics are those of bwd_attention_kernel (see dfa3d_backward.hip for the formulas and the
