@@ -625,8 +625,21 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
       TT_MARK(4);
 
       // ---------------- phase C: per-point gradients, grad_dist taps into the LDS tile ----------------
+      // LDS floating-point atomics retire about 0.3 lanes per clock per CU on this part, integer ones more
+      // than twenty times as many.  So every tap first takes a ticket from an integer counter of its tile
+      // address (the counters live where the grad_out rows were staged: the rows phase is over); the first
+      // taker of an address adds with a plain read-modify-write (no second first taker exists), and only the
+      // others (under a fifth of the taps at 256 points per pass) use the floating-point atomic afterwards.
+      int *tickets = reinterpret_cast<int *>(gstage);
+      const bool ticketed = FUSED && R * D <= PP * C && !(diag & 1024);     // uniform over the workgroup
+      if (ticketed) {
+        for (int i = tid; i < R * D; i += n_thr) tickets[i] = 0;
+        __syncthreads();
+      }
+      float gs[4] = {0, 0, 0, 0};
+      unsigned first_mask = 0;              // bit 2k / 2k+1: this thread took the first ticket of corner k's lower / upper tap
       if (live) {
-        float gs[4], s[4], ga = 0;
+        float s[4], ga = 0;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           const float dk = dots[tid * 4 + k];
@@ -656,9 +669,17 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
             if (tr[k] >= 0 && tap.inside && gs[k] != 0 && !(diag & 2)) {
-              float *dst = gd + tr[k] * D + tap.d0;
-              if (tap.lo_ok) atomicAdd(dst, tap.hd * gs[k]);
-              if (tap.hi_ok) atomicAdd(dst + 1, tap.ld * gs[k]);
+              const int at = tr[k] * D + tap.d0;
+              if (ticketed) {
+                if (tap.lo_ok && atomicAdd(&tickets[at], 1) == 0) first_mask |= 1u << (2 * k);
+                if (tap.hi_ok && atomicAdd(&tickets[at + 1], 1) == 0) first_mask |= 2u << (2 * k);
+              } else {
+                if (tap.lo_ok) atomicAdd(gd + at, tap.hd * gs[k]);
+                if (tap.hi_ok) atomicAdd(gd + at + 1, tap.ld * gs[k]);
+              }
+            } else {
+              gs[k] = (g.key[k] >= 0 && tap.inside) ? gs[k] : 0.f;      // no taps below for this corner
+              if (!(tr[k] >= 0 && tap.inside) || (diag & 2)) tr[k] = -1;
             }
             gz += (g.key[k] >= 0 && tap.inside) ? gs[k] * (hi[k] - lo[k]) : 0.f;
           }
@@ -669,6 +690,30 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           for (int k = 0; k < 4; ++k) go4[k] = gs[k];
         }
         grad_attn[gp] = ga;
+      }
+      if (ticketed) {
+        __syncthreads();                                 // every ticket taken
+        if (live) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            if (tr[k] >= 0 && gs[k] != 0) {
+              float *dst = gd + tr[k] * D + tap.d0;
+              if (first_mask & (1u << (2 * k))) dst[0] += tap.hd * gs[k];
+              if (first_mask & (2u << (2 * k))) dst[1] += tap.ld * gs[k];
+            }
+          }
+        }
+        __syncthreads();                                 // plain updates done before the atomic ones start
+        if (live) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            if (tr[k] >= 0 && gs[k] != 0) {
+              float *dst = gd + tr[k] * D + tap.d0;
+              if (tap.lo_ok && !(first_mask & (1u << (2 * k)))) atomicAdd(dst, tap.hd * gs[k]);
+              if (tap.hi_ok && !(first_mask & (2u << (2 * k)))) atomicAdd(dst + 1, tap.ld * gs[k]);
+            }
+          }
+        }
       }
       __syncthreads();                                   // before the next pass reuses the scratch arrays
       TT_MARK(5);
