@@ -815,7 +815,12 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
   const int TY = p.ty, TX = p.tx, TW = TX + 1, R = (TY + 1) * TW;
   const int tid = threadIdx.x, n_thr = blockDim.x;
   float *gd = smem;
+  // 16-bit ticket counters, one per tile address, behind the tile (see the fused kernel's phase C: integer
+  // LDS atomics are more than twenty times faster than floating-point ones).  Zero between rounds: whoever
+  // takes the first ticket of an address resets it after use.
+  uint32_t *tickets = reinterpret_cast<uint32_t *>(smem + ((R * D + 3) & ~3));
   for (int i = tid; i < R * D; i += n_thr) gd[i] = 0;
+  for (int i = tid; i < (R * D + 1) / 2; i += n_thr) tickets[i] = 0;
   const int CH = p.chunk;
   int classes_done = 0;                                   // thread 0: queues found empty so far
   for (;;) {
@@ -844,30 +849,62 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
     const int y0 = (tile / p.tiles_x[l]) * TY, x0 = (tile % p.tiles_x[l]) * TX;
     const rsrc_t dist_r = make_rsrc(dist + (size_t)b * S * M * D, (size_t)S * M * D * sizeof(T));
 
-    for (int i = tid; i < n_item; i += n_thr) {
-      const size_t gp = ws.entries[seg + i];
-      const float4 rec = ws.recs[seg + i];
-      const Point2D<float> g = locate_2d<float>(rec.x, rec.y, H, W, start);
-      const DepthTap<float> tap = locate_depth<float>(rec.z, Dd);
-      float sc[4], lo[4], hi[4];
-      corner_scores<T, float>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
-      const T *gi = grad_score + gp * 4;
-      float gz = 0;
+    // n_thr points per round (fewer than 2^16 tickets per address and round)
+    for (int base = 0; base < n_item; base += n_thr) {       // uniform over the workgroup
+      const int i = base + tid;
+      int at[4] = {-1, -1, -1, -1};                          // tile address of each corner's UPPER tap (bin d0 + 1 >= 0)
+      float gk[4] = {0, 0, 0, 0};
+      unsigned first_mask = 0;
+      DepthTap<float> tap;
+      tap.inside = tap.lo_ok = tap.hi_ok = false; tap.d0 = 0; tap.ld = tap.hd = 0;
+      if (i < n_item) {
+        const size_t gp = ws.entries[seg + i];
+        const float4 rec = ws.recs[seg + i];
+        const Point2D<float> g = locate_2d<float>(rec.x, rec.y, H, W, start);
+        tap = locate_depth<float>(rec.z, Dd);
+        float sc[4], lo[4], hi[4];
+        corner_scores<T, float>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
+        const T *gi = grad_score + gp * 4;
+        float gz = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (g.key[k] >= 0 && tap.inside) {
+            gk[k] = Elem<T>::ld(gi + k);
+            const int ry = g.h0 + (k >= 2 ? 1 : 0) - y0, rx = g.w0 + ((k == 1 || k == 2) ? 1 : 0) - x0;
+            if (ry >= 0 && ry <= TY && rx >= 0 && rx <= TX && gk[k] != 0) {
+              at[k] = (ry * TW + rx) * D + tap.d0 + 1;
+              if (tap.lo_ok) {
+                const int sh = 16 * ((at[k] - 1) & 1);
+                if (((atomicAdd(&tickets[(at[k] - 1) >> 1], 1u << sh) >> sh) & 0xFFFFu) == 0) first_mask |= 1u << (2 * k);
+              }
+              if (tap.hi_ok) {
+                const int sh = 16 * (at[k] & 1);
+                if (((atomicAdd(&tickets[at[k] >> 1], 1u << sh) >> sh) & 0xFFFFu) == 0) first_mask |= 2u << (2 * k);
+              }
+            }
+            gz += gk[k] * (hi[k] - lo[k]);
+          }
+        }
+        float *gl = grad_loc3 + gp * 3;
+        gl[0] = 0; gl[1] = 0; gl[2] = gz * (float)Dd;
+      }
+      __syncthreads();                                     // every ticket of the round taken
+      uint16_t *ticket16 = reinterpret_cast<uint16_t *>(tickets);
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        if (g.key[k] >= 0 && tap.inside) {
-          const float gk = Elem<T>::ld(gi + k);
-          const int ry = g.h0 + (k >= 2 ? 1 : 0) - y0, rx = g.w0 + ((k == 1 || k == 2) ? 1 : 0) - x0;
-          if (ry >= 0 && ry <= TY && rx >= 0 && rx <= TX && gk != 0) {
-            float *dst = gd + (ry * TW + rx) * D + tap.d0;
-            if (tap.lo_ok) atomicAdd(dst, tap.hd * gk);
-            if (tap.hi_ok) atomicAdd(dst + 1, tap.ld * gk);
-          }
-          gz += gk * (hi[k] - lo[k]);
+        if (at[k] >= 0) {
+          if (first_mask & (1u << (2 * k))) { gd[at[k] - 1] += tap.hd * gk[k]; ticket16[at[k] - 1] = 0; }
+          if (first_mask & (2u << (2 * k))) { gd[at[k]] += tap.ld * gk[k]; ticket16[at[k]] = 0; }
         }
       }
-      float *gl = grad_loc3 + gp * 3;
-      gl[0] = 0; gl[1] = 0; gl[2] = gz * (float)Dd;
+      __syncthreads();                                     // plain updates done before the atomic ones start
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (at[k] >= 0) {
+          if (tap.lo_ok && !(first_mask & (1u << (2 * k)))) atomicAdd(gd + at[k] - 1, tap.hd * gk[k]);
+          if (tap.hi_ok && !(first_mask & (2u << (2 * k)))) atomicAdd(gd + at[k], tap.ld * gk[k]);
+        }
+      }
     }
     __syncthreads();
     float *gdist_b = grad_dist + (size_t)b * S * M * D;
@@ -958,7 +995,10 @@ struct TileConfig { int ty, tx, block, pp; size_t lds; };
 
 // kind 0: both stages, 1: stage 2 alone (no depth tile), 2: stage 1 alone (depth tile only)
 static size_t tile_lds_bytes(int kind, int ty, int tx, int C, int D, int pp) {
-  if (kind == 2) return (size_t)(ty + 1) * (tx + 1) * D * 4;
+  if (kind == 2) {       // depth tile + 16-bit tickets
+    const size_t n = (size_t)(ty + 1) * (tx + 1) * D;
+    return ((n + 3) & ~(size_t)3) * 4 + ((n + 1) / 2) * 4;
+  }
   return (size_t)tile_lds_layout(ty, tx, C, kind == 1 ? 0 : D, pp).total * 4;
 }
 
