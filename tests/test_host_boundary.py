@@ -58,6 +58,18 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     assert rc == -1 and b"stride" in L.dfa3d_last_error()
     rc = L.dfa3d_ms_depth_score_sample_backward(one, one, one, one, one, null, one, null, 0, 1, 10, 8, 16, 2, 5, 4, 0, null)
     assert rc == -1 and b"grad_dist" in L.dfa3d_last_error()
+    # camera re-batching: dtype, dimensions, pointers
+    rc = L.dfa3d_rebatch_gather(one, 0, 16, one, null, one, 1, 6, 8, 16, 4, 2, null)
+    assert rc == -1 and b"dtype" in L.dfa3d_last_error()          # bf16 is not offered
+    rc = L.dfa3d_rebatch_gather(one, 0, 16, one, null, one, 1, 6, 0, 16, 4, 0, null)
+    assert rc == -1 and b"positive" in L.dfa3d_last_error()
+    rc = L.dfa3d_rebatch_gather(one, -1, 16, one, null, one, 1, 6, 8, 16, 4, 0, null)
+    assert rc == -1 and b"strides" in L.dfa3d_last_error()
+    rc = L.dfa3d_rebatch_combine(one, null, null, one, 1, 6, 8, 16, 4, 0, null)
+    assert rc == -1 and b"pos is NULL" in L.dfa3d_last_error()
+    assert L.dfa3d_fused_backward_workspace_bytes(6, 30825, 8, 32, 64, 4, 10000, 8, 1, 0) > \
+        L.dfa3d_fused_backward_workspace_bytes(6, 30825, 8, 32, 64, 4, 10000, 8, 8, 0) > 0
+    assert L.dfa3d_fused_backward_workspace_bytes(6, 30825, 8, 32, 64, 4, 10000, 8, 8, 1) == 0    # fp64: direct kernels
     assert L.dfa3d_set_tunable(b"iters", 0) == -1
     assert L.dfa3d_set_tunable(b"nope", 1) == -1
     assert L.dfa3d_set_tunable(b"iters", 1) == 0 and L.dfa3d_set_tunable(b"vec", 0) == 0
