@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 MEASURED_TRAFFIC_BYTES = {
     # profiles/fwd_attention_and_tile_backward_base_fp32.txt
     ("base", "forward"): 5.21e9,
-    ("base", "backward_tile"): 4.42e9,
+    ("base", "backward_tile"): 4.48e9,
 }
 
 
@@ -233,6 +233,19 @@ def main():
     torch.cuda.synchronize()
     fwd_api_ms = (time.perf_counter() - t0) * 1e3 / a.steps
 
+    # spread of single steps (one event pair each, outside the timed region above)
+    singles = []
+    for _ in range(max(a.steps, 10)):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        step()
+        e1.record()
+        e1.synchronize()
+        singles.append(e0.elapsed_time(e1))
+    singles.sort()
+    pick = lambda q: round(singles[min(len(singles) - 1, int(q * len(singles)))], 4)
+    step_spread = {"p10": pick(0.1), "median": pick(0.5), "p90": pick(0.9)}
+
     # ---- per-kernel durations: launches bracketed by events on the launch stream ----
     B, S, M, C = value.shape
     D = dist.shape[3]
@@ -303,6 +316,7 @@ def main():
         "config": {"workload": f"{a.workload}: B={w.B} Q={w.Q} M={w.M} C={w.C} L={w.L} "
                                f"levels={'/'.join(f'{h}x{x}' for h, x in w.levels)} D={w.D} P={w.P} "
                                f"({w.points} sampled points), one-stage Function forward+backward"},
+        "step_ms_spread": step_spread,
         "fwd_ms": round(fwd_api_ms, 4), "fwd_kernel_ms": round(fwd_ms, 4),
         "bwd_launches_ms": round(bwd_all_ms, 4), "grad_zero_fill_ms": round(fill_ms, 4),
         "fwd_points_per_s": w.points / (fwd_api_ms * 1e-3),
