@@ -268,11 +268,13 @@ __device__ __forceinline__ Point2D<A> locate_2d(A x, A y, int H, int W, int star
   Point2D<A> g;
   const A h_im = to_pixel(y, H), w_im = to_pixel(x, W);
   g.inside = h_im > -1 && w_im > -1 && h_im < H && w_im < W;
-  const int h0 = floor_index(h_im), w0 = floor_index(w_im);
+  // a point that fails the range test (NaN and infinite coordinates do) gets harmless geometry: nothing
+  // non-finite may reach a product with a masked, zero operand
+  const int h0 = g.inside ? floor_index(h_im) : 0, w0 = g.inside ? floor_index(w_im) : 0;
   g.h0 = h0;
   g.w0 = w0;
-  g.lh = h_im - h0;
-  g.lw = w_im - w0;
+  g.lh = g.inside ? h_im - h0 : (A)0;
+  g.lw = g.inside ? w_im - w0 : (A)0;
   g.hh = 1 - g.lh;
   g.hw = 1 - g.lw;
   const bool h_lo = h0 >= 0 && h0 <= H - 1, h_hi = h0 + 1 >= 0 && h0 + 1 <= H - 1;
@@ -296,9 +298,9 @@ template <typename A> __device__ __forceinline__ DepthTap<A> locate_depth(A z, i
   DepthTap<A> t;
   const A d_im = to_pixel(z, Dd);
   t.inside = d_im > -1 && d_im < Dd;
-  t.d0 = floor_index(d_im);
-  t.ld = d_im - t.d0;
-  t.hd = 1 - t.ld;
+  t.d0 = t.inside ? floor_index(d_im) : 0;
+  t.ld = t.inside ? d_im - t.d0 : (A)0;       // outside (NaN included): both weights 0, not NaN * 0
+  t.hd = t.inside ? 1 - t.ld : (A)0;
   t.lo_ok = t.inside && t.d0 >= 0 && t.d0 <= Dd - 1;
   t.hi_ok = t.inside && t.d0 + 1 >= 0 && t.d0 + 1 <= Dd - 1;
   return t;

@@ -476,6 +476,24 @@ def test_bf16_other_entry_points(oracle):
     torch.testing.assert_close(ga.cpu(), p_ga, **F32_BWD)
 
 
+def test_non_finite_and_huge_locations_are_skipped(oracle):
+    """NaN, infinite and absurdly large coordinates fail the reference's range tests (every comparison with a
+    NaN is false, cuh:69 / cuh:262) and contribute nothing; no index derived from them is ever used."""
+    dev = _dev()
+    t = tiny_case(31, C=32, M=2, Q=40, P=4, levels=((9, 11), (5, 6)), dtype=torch.float32)
+    loc = t["loc"].clone()
+    flat = loc.view(-1, 3)
+    bad = [float("nan"), float("inf"), float("-inf"), 1e30, -1e30, 3e9, -3e9]
+    for i, v in enumerate(bad * 3):
+        flat[7 * i + 3, i % 3] = v
+    inp = dict(_as_inputs(t), sampling_locations=loc)
+    got = _gpu_one_stage(inp, dev)
+    want = _oracle_one_stage(oracle, inp)
+    for g in got:
+        assert torch.isfinite(g).all()
+    _compare(got, want, F32_FWD, F32_BWD)
+
+
 def test_nan_in_unsampled_pixel_does_not_leak(oracle):
     """Corners outside the map are never read and never multiplied in."""
     dev = _dev()
