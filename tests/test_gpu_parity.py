@@ -476,6 +476,37 @@ def test_bf16_other_entry_points(oracle):
     torch.testing.assert_close(ga.cpu(), p_ga, **F32_BWD)
 
 
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32], ids=["fp64", "fp32"])
+def test_degenerate_level_shapes_and_sixteen_levels(oracle, dtype):
+    """Levels of one pixel, one row, one column; the maximum of 16 levels."""
+    dev = _dev()
+    tol = (dict(rtol=1e-10, atol=1e-11),) * 2 if dtype == torch.float64 else (F32_FWD, F32_BWD)
+    shapes = [((1, 1), (1, 5), (7, 1), (2, 2)),
+              tuple((1 + i % 3, 1 + (i * 5) % 4) for i in range(16))]
+    for i, levels in enumerate(shapes):
+        t = tiny_case(40 + i, C=8, M=2, Q=13, P=2, D=4, levels=levels, dtype=dtype)
+        inp = _as_inputs(t)
+        _compare(_gpu_one_stage(inp, dev), _oracle_one_stage(oracle, inp), *tol)
+
+
+def test_nothing_sampled_and_nothing_asked(oracle):
+    """Every location outside every map: zeros everywhere.  No queries at all: empty results, zero gradients."""
+    dev = _dev()
+    F1, _, _ = _functions()
+    t = tiny_case(50, C=32, M=2, Q=9, P=4, levels=((6, 7), (3, 3)), dtype=torch.float32, lo=1.5, hi=2.5)
+    got = _gpu_one_stage(_as_inputs(t), dev)
+    for g in got:
+        assert g.abs().max().item() == 0
+    value = t["value"].to(dev).requires_grad_()
+    dist = t["dist"].to(dev).requires_grad_()
+    loc = t["loc"][:, :0].contiguous().to(dev).requires_grad_()
+    attn = t["attn"][:, :0].contiguous().to(dev).requires_grad_()
+    out, score = F1.apply(value, dist, t["shapes3"].to(dev), t["lsi"].to(dev), loc, attn, 64)
+    assert out.shape == (2, 0, 64) and score.shape == (2, 0, 2, 2, 4, 4)
+    gv, gd, gl, ga = torch.autograd.grad(out, [value, dist, loc, attn], torch.zeros_like(out))
+    assert gv.abs().max().item() == 0 and gd.abs().max().item() == 0 and gl.numel() == 0 and ga.numel() == 0
+
+
 def test_non_finite_and_huge_locations_are_skipped(oracle):
     """NaN, infinite and absurdly large coordinates fail the reference's range tests (every comparison with a
     NaN is false, cuh:69 / cuh:262) and contribute nothing; no index derived from them is ever used."""
