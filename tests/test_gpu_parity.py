@@ -412,6 +412,33 @@ def test_bf16_storage(oracle):
     torch.testing.assert_close(ga.cpu(), o_ga, **F32_BWD)
 
 
+@pytest.mark.parametrize("case", [dict(seed=60, C=6, M=3, Q=17, P=3, D=5, levels=((7, 5), (3, 4))),
+                                  dict(seed=61, C=16, M=2, Q=9, P=5, D=7, levels=((4, 9),)),
+                                  dict(seed=62, C=1, M=2, Q=5, P=2, D=2, levels=((3, 3), (2, 2)))],
+                         ids=lambda c: f"seed{c['seed']}")
+def test_bf16_odd_shapes(oracle, case):
+    """bfloat16 storage with row lengths that rule out the aligned vector loads (odd D, C = 1 / 6 / 16)."""
+    dev = _dev()
+    F1, _, _ = _functions()
+    t = tiny_case(dtype=torch.float32, **case)
+    inp = _as_inputs(t)
+    r16 = dict(inp, value=inp["value"].bfloat16().float(), value_dpt_dist=inp["value_dpt_dist"].bfloat16().float(),
+               grad_output=inp["grad_output"].bfloat16().float())
+    value = inp["value"].bfloat16().to(dev).requires_grad_()
+    dist = inp["value_dpt_dist"].bfloat16().to(dev).requires_grad_()
+    loc, attn = inp["sampling_locations"].to(dev).requires_grad_(), inp["attention_weights"].to(dev).requires_grad_()
+    out, score = F1.apply(value, dist, inp["spatial_shapes"].to(dev), inp["level_start_index"].to(dev), loc, attn, 64)
+    gv, gd, gl, ga = torch.autograd.grad(out, [value, dist, loc, attn], inp["grad_output"].bfloat16().to(dev))
+    o_out, o_score, o_gv, o_gd, o_gl, o_ga = _oracle_one_stage(oracle, r16)
+    bf = dict(rtol=8e-3, atol=8e-3)
+    torch.testing.assert_close(out.float().cpu(), o_out, **bf)
+    torch.testing.assert_close(score.float().cpu(), o_score, **bf)
+    torch.testing.assert_close(gv.float().cpu(), o_gv, **bf)
+    torch.testing.assert_close(gd.float().cpu(), o_gd, rtol=8e-3, atol=8e-3 * max(1.0, o_gd.abs().max().item()))
+    torch.testing.assert_close(gl.cpu(), o_gl, **F32_BWD)
+    torch.testing.assert_close(ga.cpu(), o_ga, **F32_BWD)
+
+
 def test_bf16_other_entry_points(oracle):
     """bfloat16 storage through the two separate stages, through the shared-distribution / weight_update
     Function and through plain deformable attention, same bounds as test_bf16_storage."""
