@@ -67,8 +67,7 @@ struct BinWorkspace {      // device pointers into the caller's workspace
   int *queues;             // kClasses counters, kQueueStride ints apart
   int *counts;             // points per bin
   int *cursor;             // begin of each bin's segment after the scan, end after the fill
-  int *chunk_end;          // inclusive prefix of work items per bin
-  int *item_bin;           // bin of each work item
+  int4 *items;             // work items: (bin, begin of its points, number of points, work items of the bin)
   uint32_t *entries;       // point indices grouped by bin
   float4 *recs;            // (x, y, z, attention weight) of the same points, same order
 };
@@ -244,10 +243,10 @@ __global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws) {
       if (i < n) {
         if (i % per_class == 0) ws.plan->class_start[i / per_class] = run_c;
         ws.cursor[i] = run_p;
+        for (int t = 0; t < k[j]; ++t)
+          ws.items[run_c + t] = make_int4(i, run_p + t * ch, min(ch, c[j] - t * ch), k[j]);
         run_p += c[j];
-        for (int t = 0; t < k[j]; ++t) ws.item_bin[run_c + t] = i;
         run_c += k[j];
-        ws.chunk_end[i] = run_c;
       }
     }
     __syncthreads();                                         // everyone has read the carry and the wave sums
@@ -324,6 +323,27 @@ __device__ __forceinline__ int pop_item(const BinWorkspace &ws, const BinPlan &p
   return -1;
 }
 
+// Thread 0's pipeline of work items: the item taken now was popped two items ago and its record requested
+// one item ago, so neither the queue atomic nor the record's load is waited for.
+struct ItemFetch {
+  int classes_done, w_next;
+  int4 rec;
+  __device__ __forceinline__ int4 load(const BinWorkspace &ws, int w) const {
+    return w >= 0 ? ws.items[w] : make_int4(-1, 0, 0, 0);
+  }
+  __device__ __forceinline__ void start(const BinWorkspace &ws, const BinPlan &p, int home) {
+    classes_done = 0;
+    const int w = pop_item(ws, p, home, classes_done);
+    rec = load(ws, w);
+    w_next = w >= 0 ? pop_item(ws, p, home, classes_done) : -1;
+  }
+  __device__ __forceinline__ void advance(const BinWorkspace &ws, const BinPlan &p, int home, int4 *out) {
+    *out = rec;
+    rec = load(ws, w_next);
+    w_next = w_next >= 0 ? pop_item(ws, p, home, classes_done) : -1;
+  }
+};
+
 struct RowTask { float w; uint32_t who; };   // who = point slot * 4 + corner: the index of the task's dot
 
 __device__ __forceinline__ float dpp_xadd(float x, int pick) {
@@ -397,7 +417,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
   // Md: heads stored in dist (M, or 1 = shared by all heads); Mg: heads of the grad_dist buffer written here
   constexpr int RPI = kWave / LPR;                  // row groups per wavefront
   extern __shared__ __align__(16) float smem[];
-  __shared__ int s_bin, s_item;
+  __shared__ int4 s_item;
 
   const BinPlan &p = *ws.plan;
   const int nb = p.bins_per_bm;
@@ -419,26 +439,17 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
   for (int i = tid; i < R * (C + D); i += n_thr) smem[i] = 0;   // gv and gd are adjacent
   TT_DECL
 
-  const int CH = p.chunk;
-  int classes_done = 0;                                   // thread 0: queues found empty so far
+  ItemFetch fetch;
+  if (tid == 0) fetch.start(ws, p, blockIdx.x % kClasses);
   for (;;) {
     // ---- next work item: (bin, chunk of its points), in bin order
     __syncthreads();
-    if (tid == 0) {
-      const int w = pop_item(ws, p, blockIdx.x % kClasses, classes_done);
-      s_bin = w >= 0 ? ws.item_bin[w] : -1;
-      s_item = w;
-    }
+    if (tid == 0) fetch.advance(ws, p, blockIdx.x % kClasses, &s_item);
     __syncthreads();
-    const int bin = s_bin;
-    if (bin < 0) break;                                   // queue drained: every wave leaves
+    const int4 item = s_item;
+    const int bin = item.x, seg = item.y, n_item = item.z, chunks_here = item.w;
+    if (bin < 0) break;                                   // queues drained: every wave leaves
     TT_MARK(0);
-    const int n_bin = ws.counts[bin];
-    const int chunks_here = (n_bin + CH - 1) / CH;
-    const int chunk_id = s_item - (ws.chunk_end[bin] - chunks_here);
-    const int first = chunk_id * CH;
-    const int n_item = min(CH, n_bin - first);
-    const int seg = ws.cursor[bin] - n_bin + first;       // the fill advanced the cursor to the segment's end
     const int bm = bin / nb, local = bin - bm * nb;
     int b, m;
     slot_decode(bm, B, M, b, m);
@@ -808,7 +819,7 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
     BinWorkspace ws, const T *__restrict__ dist, const T *__restrict__ grad_score, float *__restrict__ grad_dist,
     float *__restrict__ grad_loc3, int B, int S, int M, int D, int L, int Q, int P) {
   extern __shared__ __align__(16) float smem[];
-  __shared__ int s_bin, s_item;
+  __shared__ int4 s_item;
   const BinPlan &p = *ws.plan;
   const int nb = p.bins_per_bm;
   if (nb == 0) return;
@@ -821,24 +832,15 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
   uint32_t *tickets = reinterpret_cast<uint32_t *>(smem + ((R * D + 3) & ~3));
   for (int i = tid; i < R * D; i += n_thr) gd[i] = 0;
   for (int i = tid; i < (R * D + 1) / 2; i += n_thr) tickets[i] = 0;
-  const int CH = p.chunk;
-  int classes_done = 0;                                   // thread 0: queues found empty so far
+  ItemFetch fetch;
+  if (tid == 0) fetch.start(ws, p, blockIdx.x % kClasses);
   for (;;) {
     __syncthreads();
-    if (tid == 0) {
-      const int w = pop_item(ws, p, blockIdx.x % kClasses, classes_done);
-      s_bin = w >= 0 ? ws.item_bin[w] : -1;
-      s_item = w;
-    }
+    if (tid == 0) fetch.advance(ws, p, blockIdx.x % kClasses, &s_item);
     __syncthreads();
-    const int bin = s_bin;
-    if (bin < 0) break;                                   // queue drained: every wave leaves
-    const int n_bin = ws.counts[bin];
-    const int chunks_here = (n_bin + CH - 1) / CH;
-    const int chunk_id = s_item - (ws.chunk_end[bin] - chunks_here);
-    const int first = chunk_id * CH;
-    const int n_item = min(CH, n_bin - first);
-    const int seg = ws.cursor[bin] - n_bin + first;
+    const int4 item = s_item;
+    const int bin = item.x, seg = item.y, n_item = item.z;
+    if (bin < 0) break;                                   // queues drained: every wave leaves
     const int bm = bin / nb, local = bin - bm * nb;
     int b, m;
     slot_decode(bm, B, M, b, m);
@@ -967,7 +969,7 @@ __global__ __launch_bounds__(256) void head_sum_kernel(const float *__restrict__
     }
   }
 }
-struct BinLayout { size_t plan, queues, counts, cursor, chunk_end, item_bin, entries, recs, gd_heads, total; };
+struct BinLayout { size_t plan, queues, counts, cursor, items, entries, recs, gd_heads, total; };
 static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
   BinLayout o;
   const size_t nbins = (size_t)max_bins_per_bm(a.S, a.L, ty, tx) * slot_count(a.B, a.M);
@@ -977,10 +979,9 @@ static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
   o.queues = up(o.plan + sizeof(BinPlan));
   o.counts = up(o.queues + kQueueInts * sizeof(int));
   o.cursor = up(o.counts + nbins * sizeof(int));
-  o.chunk_end = up(o.cursor + nbins * sizeof(int));
   // work items: at most one partial chunk per bin plus the full chunks
-  o.item_bin = up(o.chunk_end + nbins * sizeof(int));
-  o.entries = up(o.item_bin + (nbins + npts / kMinChunk + 1) * sizeof(int));
+  o.items = up(o.cursor + nbins * sizeof(int));
+  o.entries = up(o.items + (nbins + npts / kMinChunk + 1) * sizeof(int4));
   o.recs = up(o.entries + npts * sizeof(uint32_t));
   // a distribution shared by the heads: grad_dist per head first (stores, as with a distribution per head),
   // summed over the heads afterwards; eight XCDs adding atomically into one shared tile cost twice as much
@@ -1110,8 +1111,7 @@ static BinWorkspace carve_workspace(void *workspace, const BinLayout &lay) {
   ws.queues = reinterpret_cast<int *>(base + lay.queues);
   ws.counts = reinterpret_cast<int *>(base + lay.counts);
   ws.cursor = reinterpret_cast<int *>(base + lay.cursor);
-  ws.chunk_end = reinterpret_cast<int *>(base + lay.chunk_end);
-  ws.item_bin = reinterpret_cast<int *>(base + lay.item_bin);
+  ws.items = reinterpret_cast<int4 *>(base + lay.items);
   ws.entries = reinterpret_cast<uint32_t *>(base + lay.entries);
   ws.recs = reinterpret_cast<float4 *>(base + lay.recs);
   return ws;
