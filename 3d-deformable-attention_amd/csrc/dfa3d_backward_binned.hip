@@ -323,6 +323,18 @@ __device__ __forceinline__ int pop_item(const BinWorkspace &ws, const BinPlan &p
   return -1;
 }
 
+// Inclusive prefix sum over the 64 lanes with DPP moves: shifts by 1, 2, 4, 8 inside rows of 16 lanes, then
+// lane 15 of a row to the next row, then lane 31 to the upper half.
+__device__ __forceinline__ int wave_inclusive_scan(int x) {
+  x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, false);   // row_shr:1
+  x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, false);   // row_shr:2
+  x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, false);   // row_shr:4
+  x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, false);   // row_shr:8
+  x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false);   // row_bcast:15 into rows 1 and 3
+  x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);   // row_bcast:31 into rows 2 and 3
+  return x;
+}
+
 // Thread 0's pipeline of work items: the item taken now was popped two items ago and its record requested
 // one item ago, so neither the queue atomic nor the record's load is waited for.
 struct ItemFetch {
@@ -525,23 +537,21 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
       }
       __syncthreads();                                   // counts complete
       TT_MARK(2);
-      if (wave == 0) {                                   // exclusive prefix of the row counters
+      // Exclusive prefix of the row counters.  Every wavefront that places tasks computes it, two rows per
+      // lane and 128 rows per step, and writes the same numbers: it can go on with its own copy without
+      // waiting for the others.
+      if (wave * kWave < PP) {
         int run = 0;
-        for (int r0 = 0; r0 < R; r0 += kWave) {
-          const int r = r0 + lane;
-          const int c = r < R ? cnt[r] : 0;
-          int inc = c;
-#pragma unroll
-          for (int off = 1; off < kWave; off <<= 1) {
-            const int up = __shfl_up(inc, off, kWave);
-            if (lane >= off) inc += up;
-          }
-          if (r < R) offs[r] = run + inc - c;
-          run += __shfl(inc, kWave - 1, kWave);
+        for (int r0 = 0; r0 < R; r0 += 2 * kWave) {
+          const int r = r0 + 2 * lane;
+          const int c0 = r < R ? cnt[r] : 0, c1 = r + 1 < R ? cnt[r + 1] : 0;
+          const int inc = wave_inclusive_scan(c0 + c1);
+          if (r < R) offs[r] = run + inc - c0 - c1;
+          if (r + 1 < R) offs[r + 1] = run + inc - c1;
+          run += __builtin_amdgcn_readlane(inc, kWave - 1);
         }
         if (lane == 0) offs[R] = run;
       }
-      __syncthreads();
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         if (tid >= PP) {
