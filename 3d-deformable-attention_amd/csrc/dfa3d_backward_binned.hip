@@ -453,6 +453,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
 
   ItemFetch fetch;
   if (tid == 0) fetch.start(ws, p, blockIdx.x % kClasses);
+  int pass_tag = 0x5EED0000;                               // changes with every pass of this workgroup
   for (;;) {
     // ---- next work item: (bin, chunk of its points), in bin order
     __syncthreads();
@@ -647,16 +648,15 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
 
       // ---------------- phase C: per-point gradients, grad_dist taps into the LDS tile ----------------
       // LDS floating-point atomics retire about 0.3 lanes per clock per CU on this part, integer ones more
-      // than twenty times as many.  So every tap first takes a ticket from an integer counter of its tile
-      // address (the counters live where the grad_out rows were staged: the rows phase is over); the first
-      // taker of an address adds with a plain read-modify-write (no second first taker exists), and only the
-      // others (under a fifth of the taps at 256 points per pass) use the floating-point atomic afterwards.
+      // than twenty times as many.  So every tap first swaps this pass's tag into a word that belongs to its
+      // tile address (the words live where the grad_out rows were staged: the rows phase is over).  Whoever
+      // gets something else than the tag back is the first at that address and adds at once with a plain
+      // read-modify-write: nobody else touches the address before the barrier below.  Only the others (under
+      // a fifth of the taps at 256 points per pass) use the floating-point atomic, after that barrier.  Stale
+      // words cannot do harm: one that happens to equal the tag just sends its address's taps to the atomics.
       int *tickets = reinterpret_cast<int *>(gstage);
       const bool ticketed = FUSED && R * D <= PP * C && !(diag & 1024);     // uniform over the workgroup
-      if (ticketed) {
-        for (int i = tid; i < R * D; i += n_thr) tickets[i] = 0;
-        __syncthreads();
-      }
+      ++pass_tag;
       float gs[4] = {0, 0, 0, 0};
       unsigned first_mask = 0;              // bit 2k / 2k+1: this thread took the first ticket of corner k's lower / upper tap
       if (live) {
@@ -692,8 +692,14 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
             if (tr[k] >= 0 && tap.inside && gs[k] != 0 && !(diag & 2)) {
               const int at = tr[k] * D + tap.d0;
               if (ticketed) {
-                if (tap.lo_ok && atomicAdd(&tickets[at], 1) == 0) first_mask |= 1u << (2 * k);
-                if (tap.hi_ok && atomicAdd(&tickets[at + 1], 1) == 0) first_mask |= 2u << (2 * k);
+                if (tap.lo_ok && atomicExch(&tickets[at], pass_tag) != pass_tag) {
+                  first_mask |= 1u << (2 * k);
+                  gd[at] += tap.hd * gs[k];
+                }
+                if (tap.hi_ok && atomicExch(&tickets[at + 1], pass_tag) != pass_tag) {
+                  first_mask |= 2u << (2 * k);
+                  gd[at + 1] += tap.ld * gs[k];
+                }
               } else {
                 if (tap.lo_ok) atomicAdd(gd + at, tap.hd * gs[k]);
                 if (tap.hi_ok) atomicAdd(gd + at + 1, tap.ld * gs[k]);
@@ -713,17 +719,6 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         grad_attn[gp] = ga;
       }
       if (ticketed) {
-        __syncthreads();                                 // every ticket taken
-        if (live) {
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            if (tr[k] >= 0 && gs[k] != 0) {
-              float *dst = gd + tr[k] * D + tap.d0;
-              if (first_mask & (1u << (2 * k))) dst[0] += tap.hd * gs[k];
-              if (first_mask & (2u << (2 * k))) dst[1] += tap.ld * gs[k];
-            }
-          }
-        }
         __syncthreads();                                 // plain updates done before the atomic ones start
         if (live) {
 #pragma unroll
