@@ -731,9 +731,11 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           }
         }
       }
-      __syncthreads();                                   // before the next pass reuses the scratch arrays
+      // no barrier here: what the next pass writes before its first barrier (row counters, grad_out offsets)
+      // was last read before this pass's later barriers
       TT_MARK(5);
     }
+    __syncthreads();                                     // the tile is complete
 
     // ---------------- flush the tile (and leave it zeroed for the next item) ----------------
     float *gvalue_b = grad_value + (size_t)b * S * M * C;
