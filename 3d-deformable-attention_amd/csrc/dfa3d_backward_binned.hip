@@ -500,6 +500,9 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         g = locate_2d<float>(rec.x, rec.y, H, W, start);
         if (FUSED) {
           tap = locate_depth<float>(rec.z, Dd);
+#ifdef DFA3D_EXPERIMENT
+          if (diag & 32) { for (int k = 0; k < 4; ++k) { sc[k] = 0.5f; lo[k] = 0.1f; hi[k] = 0.2f; } } else   // cost of the depth taps
+#endif
           corner_scores<T, float>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
         } else {
           const T *si = score_in + gp * 4;
@@ -532,6 +535,9 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         for (int j = 0; j < stage_per_wave; j += RPI) {
           const int slot = wave * stage_per_wave + j + lane / LPR;
           float gg[VEC];
+#ifdef DFA3D_EXPERIMENT
+          if (diag & 256) { for (int i = 0; i < VEC; ++i) gg[i] = 1.f; } else   // cost of the grad_out loads
+#endif
           RowVec<T, float, VEC>::ld(go_r, goff[slot] + chan_off, gg);
           if (chan < C) LdsVec<VEC>::st(gstage + slot * C + chan, gg);
         }
@@ -599,6 +605,9 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
             const bool ld_ok = rn < R && offs[min(rn, R - 1) + 1] > offs[min(rn, R - 1)] && yn < H && xn < W && !(diag & 8);
             RowVec<T, float, VEC>::ld(value_r, (ld_ok ? (uint32_t)(((start + yn * W + xn) * M + m) * C * (int)sizeof(T)) : kNoRow) + chan_off, v_next);
           }
+#ifdef DFA3D_EXPERIMENT
+          if (diag & 16) n_max = 0;                      // cost of the task loop
+#endif
           if (n_max == 0) continue;                      // wave-uniform
           // tasks in flight per group: registers decide (measured: 4 with four channels per lane, 1 with eight;
           // one more costs 1 % .. 10 % of the kernel's time)
@@ -659,7 +668,11 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
       ++pass_tag;
       float gs[4] = {0, 0, 0, 0};
       unsigned first_mask = 0;              // bit 2k / 2k+1: this thread took the first ticket of corner k's lower / upper tap
+#ifdef DFA3D_EXPERIMENT
+      if (live && !(diag & 512)) {                       // cost of phase C
+#else
       if (live) {
+#endif
         float s[4], ga = 0;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -687,30 +700,37 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
             for (int k = 0; k < 4; ++k) gs[k] += gw * a;
           }
           float gz = 0;
+          int at8[8];                               // tile address of each of the eight taps, -1 = no tap
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
-            if (tr[k] >= 0 && tap.inside && gs[k] != 0 && !(diag & 2)) {
-              const int at = tr[k] * D + tap.d0;
-              if (ticketed) {
-                if (tap.lo_ok && atomicExch(&tickets[at], pass_tag) != pass_tag) {
-                  first_mask |= 1u << (2 * k);
-                  gd[at] += tap.hd * gs[k];
-                }
-                if (tap.hi_ok && atomicExch(&tickets[at + 1], pass_tag) != pass_tag) {
-                  first_mask |= 2u << (2 * k);
-                  gd[at + 1] += tap.ld * gs[k];
-                }
-              } else {
-                if (tap.lo_ok) atomicAdd(gd + at, tap.hd * gs[k]);
-                if (tap.hi_ok) atomicAdd(gd + at + 1, tap.ld * gs[k]);
-              }
-            } else {
+            const bool taps = tr[k] >= 0 && tap.inside && gs[k] != 0 && !(diag & 2);
+            const int at = tr[k] * D + tap.d0;
+            at8[2 * k] = (taps && tap.lo_ok) ? at : -1;
+            at8[2 * k + 1] = (taps && tap.hi_ok) ? at + 1 : -1;
+            if (!taps) {
               gs[k] = (g.key[k] >= 0 && tap.inside) ? gs[k] : 0.f;      // no taps below for this corner
               if (!(tr[k] >= 0 && tap.inside) || (diag & 2)) tr[k] = -1;
             }
             gz += (g.key[k] >= 0 && tap.inside) ? gs[k] * (hi[k] - lo[k]) : 0.f;
           }
           gl[2] = gz * (float)Dd;
+          if (ticketed) {
+            // the eight swaps back to back, then the reads of the first takers, then their writes: one LDS
+            // round trip each instead of one per tap (a thread's eight addresses are all different)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              if (at8[j] >= 0 && atomicExch(&tickets[at8[j]], pass_tag) != pass_tag) first_mask |= 1u << j;
+            float cur8[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) cur8[j] = (first_mask >> j & 1) ? gd[at8[j]] : 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              if (first_mask >> j & 1) gd[at8[j]] = cur8[j] + ((j & 1) ? tap.ld : tap.hd) * gs[j >> 1];
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              if (at8[j] >= 0) atomicAdd(gd + at8[j], ((j & 1) ? tap.ld : tap.hd) * gs[j >> 1]);
+          }
         } else if (grad_score_out != nullptr) {
           float *go4 = grad_score_out + gp * 4;
 #pragma unroll
