@@ -315,8 +315,10 @@ __device__ __forceinline__ int pop_item(const BinWorkspace &ws, const BinPlan &p
     const int c = (home + classes_done) % kClasses;
     const int lo = p.class_start[c], hi = p.class_start[c + 1];
     if (lo < hi) {
-      const int w = lo + atomicAdd(&ws.queues[c * kQueueStride], 1);
-      if (w < hi) return w;
+      // from the end: the bins of the coarsest level, which hold the most points, come last in a (batch, head)
+      // and should not be what the kernel's last workgroups are left with
+      const int w = hi - 1 - atomicAdd(&ws.queues[c * kQueueStride], 1);
+      if (w >= lo) return w;
     }
     ++classes_done;
   }
@@ -961,6 +963,10 @@ static int max_bins_per_bm(int S, int L, int ty, int tx) {
 }
 
 constexpr int kMinChunk = 64;        // smallest accepted points-per-item
+// Points of a bin per work item.  A bin that fits one item is flushed with stores instead of atomic adds, so
+// large items pay; the queues are served from their ends so that the heavy bins of the coarse levels do not
+// come last.  Measured at the BEVFormer-base shape: 1024 -> 2.01 ms, 2048 -> 1.87, 4096 -> 1.83, 8192 -> 1.92.
+constexpr int kDefaultChunk = 4096;
 // only the fused entry point sets dist_heads
 static bool shared_dist(const BwdArgs &a) { return a.dist_heads == 1 && a.M > 1; }
 
@@ -1149,7 +1155,7 @@ static BinWorkspace carve_workspace(void *workspace, const BinLayout &lay) {
 static hipError_t run_binning(const BwdArgs &a, const BinWorkspace &ws, int ty, int tx, hipStream_t stream) {
   const int mb = max_bins_per_bm(a.S, a.L, ty, tx);
   hipLaunchKernelGGL(plan_and_clear_kernel, dim3(64), dim3(256), 0, stream, ws, a.shapes, a.shape_stride, a.level_start,
-                     a.L, a.S, (a.dist != nullptr || a.C == 0) ? a.D : 0, a.B, a.M, ty, tx, a.chunk_hint > 0 ? a.chunk_hint : 1024, mb);
+                     a.L, a.S, (a.dist != nullptr || a.C == 0) ? a.D : 0, a.B, a.M, ty, tx, a.chunk_hint > 0 ? a.chunk_hint : kDefaultChunk, mb);
   const int q_blocks = (a.Q + kBinQueries - 1) / kBinQueries;
   const long long blocks = (long long)a.B * a.M * q_blocks;
   if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;

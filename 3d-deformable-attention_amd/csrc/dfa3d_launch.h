@@ -71,7 +71,7 @@ struct BwdArgs {
   int diag;                          // measurement aid: bit 0 drops the grad_value updates, bit 1 the grad_dist updates
   int tile_hint;                     // binned path: tile edge as ty * 100 + tx (0 = automatic)
   int block_hint;                    // binned path: threads per tile workgroup (0 = 256)
-  int chunk_hint;                    // binned path: points of a bin per work item (0 = 1024)
+  int chunk_hint;                    // binned path: points of a bin per work item (0 = 4096)
   int pass_hint;                     // binned path: points per pass, 128 or 256 (0 = 256)
   int stage;                         // binned path, measurement aid: 0 all kernels, 1 binning only, 2 tile kernel only
 };

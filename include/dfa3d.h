@@ -175,7 +175,7 @@ const char *dfa3d_last_error(void);
  *   "tile"   binned backward: tile edge in pixels as ty*100+tx, 0 = automatic
  *   "block"  binned backward: threads per tile workgroup, 256 or 0/512
  *   "pass"   binned backward: points a tile workgroup takes per pass, 128 or 0/256
- *   "chunk"  binned backward: points of one tile handled by one work item, 0 = 1024
+ *   "chunk"  binned backward: points of one tile handled by one work item, 0 = 4096
  *   "bwd_stage" measurement aid for the binned backward: 0 = every kernel, 1 = the binning kernels
  *            only, 2 = the tile kernel only (on a workspace a stage-1 call has just prepared) */
 int dfa3d_set_tunable(const char *name, int value);
