@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 MEASURED_TRAFFIC_BYTES = {
     # profiles/fwd_attention_and_tile_backward_base_fp32.txt
     ("base", "forward"): 5.21e9,
-    ("base", "backward_tile"): 4.48e9,
+    ("base", "backward_tile"): 4.31e9,
 }
 
 
