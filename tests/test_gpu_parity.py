@@ -534,6 +534,19 @@ def test_nothing_sampled_and_nothing_asked(oracle):
     assert gv.abs().max().item() == 0 and gd.abs().max().item() == 0 and gl.numel() == 0 and ga.numel() == 0
 
 
+def test_every_point_in_one_pixel_cell(oracle):
+    """All sampling points in the same pixel cell and depth interval: one tile gets everything (several work
+    items for one bin, every tile address contested).  Sums of 12 000 float32 terms: looser tolerance."""
+    dev = _dev()
+    t = tiny_case(55, B=1, C=32, M=2, Q=1500, P=4, D=16, levels=((20, 30),), dtype=torch.float32)
+    g = torch.Generator().manual_seed(5)
+    loc = torch.tensor([0.37, 0.52, 0.41]) + (torch.rand(t["loc"].shape, generator=g) - 0.5) * 0.01
+    inp = dict(_as_inputs(t), sampling_locations=loc.contiguous())
+    got = _gpu_one_stage(inp, dev)
+    want = _oracle_one_stage(oracle, inp)
+    _compare(got, want, F32_FWD, dict(rtol=2e-3, atol=2e-3))
+
+
 def test_non_finite_and_huge_locations_are_skipped(oracle):
     """NaN, infinite and absurdly large coordinates fail the reference's range tests (every comparison with a
     NaN is false, cuh:69 / cuh:262) and contribute nothing; no index derived from them is ever used."""
