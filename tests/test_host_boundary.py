@@ -154,7 +154,7 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
 
 
 def test_workload_byte_model_matches_published_table():
-    """Algorithmic bytes of the five benchmark configurations (MB as quoted in BASELINE.md)."""
+    """Algorithmic bytes of the benchmark configurations against hand-computed MB figures."""
     from dfa3D.workloads import WORKLOADS
     w = WORKLOADS["base"]
     assert w.S == 30825 and w.points == 15_360_000 and w.level_start_index() == [0, 23200, 29000, 30450]
