@@ -95,6 +95,28 @@ FP32_EXTRA = [
 ]
 
 
+def _random_case(seed):
+    """A shape drawn from a seeded generator: odd channel counts, head counts that are no multiple of the
+    eight XCD classes, one to five levels of unrelated sizes (maps smaller than a tile, maps of many tiles)."""
+    import random
+    r = random.Random(seed)
+    L = r.randint(1, 5)
+    levels = tuple((r.randint(1, 40), r.randint(1, 40)) for _ in range(L))
+    return dict(seed=seed, B=r.randint(1, 3), M=r.choice([1, 2, 3, 4, 6, 8, 9, 16]),
+                C=r.choice([1, 4, 8, 12, 16, 24, 32, 40, 64, 72, 128]), D=r.choice([1, 2, 3, 8, 17, 32, 64, 80]),
+                Q=r.randint(1, 400), P=r.randint(1, 9), levels=levels, lo=r.choice([0.0, -0.2]), hi=r.choice([1.0, 1.2]))
+
+
+@pytest.mark.parametrize("seed", range(100, 124))
+def test_fp32_random_shapes_match_checker(oracle, seed):
+    dev = _dev()
+    case = _random_case(seed)
+    print("case", case, flush=True)
+    t = tiny_case(**case)
+    inp = {k: (v.float() if v.is_floating_point() else v) for k, v in _as_inputs(t).items()}
+    _compare(_gpu_one_stage(inp, dev), _oracle_one_stage(oracle, inp), F32_FWD, F32_BWD)
+
+
 @pytest.mark.parametrize("case", TINY + FP32_EXTRA, ids=lambda c: f"seed{c['seed']}")
 def test_fp32_one_stage_matches_checker_tiny(oracle, case):
     dev = _dev()
@@ -327,6 +349,33 @@ def test_fp32_two_stage_workloads_match_checker(oracle, binned, sliced):
             _compare(_gpu_two_stage(inp, dev, sliced), _oracle_one_stage(oracle, inp), F32_FWD, F32_BWD)
     finally:
         _lib.set_tunable("binned", 1)
+
+
+@pytest.mark.parametrize("seed", range(130, 142))
+def test_fp32_random_shapes_two_stage_and_shared_distribution(oracle, seed):
+    """The drawn shapes of _random_case through the two separate stages (3-wide and sliced operands) and
+    through the shared-distribution Function with a gradient at weight_update."""
+    from dfa3D.functional import MultiScale3DDeformableAttnWeightUpdateFunction
+    dev = _dev()
+    case = _random_case(seed)
+    print("case", case, flush=True)
+    t = tiny_case(**case)
+    inp = {k: (v.float() if v.is_floating_point() else v) for k, v in _as_inputs(t).items()}
+    want = _oracle_one_stage(oracle, inp)
+    _compare(_gpu_two_stage(inp, dev, sliced=seed % 2 == 0), want, F32_FWD, F32_BWD)
+
+    shared = dict(inp)
+    shared["value_dpt_dist"] = inp["value_dpt_dist"][:, :, :1].contiguous()
+    g = torch.Generator().manual_seed(seed)
+    grad_wu = torch.randn(*inp["attention_weights"].shape[:3], 1, generator=g)
+    want = _shared_dist_expectation(oracle, shared, grad_wu=grad_wu)
+    v, d, loc, a = [shared[k].to(dev).requires_grad_() for k in ("value", "value_dpt_dist", "sampling_locations",
+                                                                  "attention_weights")]
+    out, wu = MultiScale3DDeformableAttnWeightUpdateFunction.apply(
+        v, d, shared["spatial_shapes"].to(dev), shared["level_start_index"].to(dev), loc, a, 64)
+    grads = torch.autograd.grad([out, wu], [v, d, loc, a], [shared["grad_output"].to(dev), grad_wu.to(dev)])
+    torch.testing.assert_close(wu.detach().cpu(), want[2], **F32_FWD)
+    _compare([out.detach().cpu(), want[1], *[x.cpu() for x in grads]], [want[0], want[1], *want[3:]], F32_FWD, F32_BWD)
 
 
 def test_fp32_base_shape_two_stage_matches_checker(oracle):
