@@ -583,6 +583,15 @@ def test_nothing_sampled_and_nothing_asked(oracle):
     assert gv.abs().max().item() == 0 and gd.abs().max().item() == 0 and gl.numel() == 0 and ga.numel() == 0
 
 
+def test_more_tiles_than_the_block_histogram_holds(oracle):
+    """A 760 x 700 map has 8360 tiles per (batch, head): more than the binning blocks count in LDS, so they
+    count in device memory."""
+    dev = _dev()
+    t = tiny_case(56, B=1, C=4, M=2, Q=3000, P=4, D=2, levels=((760, 700), (3, 5)), dtype=torch.float32)
+    inp = _as_inputs(t)
+    _compare(_gpu_one_stage(inp, dev), _oracle_one_stage(oracle, inp), F32_FWD, F32_BWD)
+
+
 def test_every_point_in_one_pixel_cell(oracle):
     """All sampling points in the same pixel cell and depth interval: one tile gets everything (several work
     items for one bin, every tile address contested).  Sums of 12 000 float32 terms: looser tolerance."""
