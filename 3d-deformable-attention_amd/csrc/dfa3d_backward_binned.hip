@@ -688,7 +688,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const float gx = (float)W * a * (g.hh * (s[1] - s[0]) + g.lh * (s[2] - s[3]));
         const float gy = (float)H * a * (g.hw * (s[3] - s[0]) + g.lw * (s[2] - s[1]));
         float *gl = grad_loc + gp * gl_stride;
-        gl[0] = gx; gl[1] = gy;
+        if (!FUSED) { gl[0] = gx; gl[1] = gy; }
         if (FUSED) {
           if (grad_score_in != nullptr) {
             const T *gi = grad_score_in + gp * 4;
@@ -715,7 +715,8 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
             }
             gz += (g.key[k] >= 0 && tap.inside) ? gs[k] * (hi[k] - lo[k]) : 0.f;
           }
-          gl[2] = gz * (float)Dd;
+          gl[0] = gx; gl[1] = gy; gl[2] = gz * (float)Dd;      // one 12-byte store
+          grad_attn[gp] = ga;                       // all stores before the tile updates: they complete slowly
           if (ticketed) {
             // the eight swaps back to back, then the reads of the first takers, then their writes: one LDS
             // round trip each instead of one per tap (a thread's eight addresses are all different)
@@ -737,8 +738,10 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           float *go4 = grad_score_out + gp * 4;
 #pragma unroll
           for (int k = 0; k < 4; ++k) go4[k] = gs[k];
+          grad_attn[gp] = ga;
+        } else {
+          grad_attn[gp] = ga;
         }
-        grad_attn[gp] = ga;
       }
       if (ticketed) {
         __syncthreads();                                 // plain updates done before the atomic ones start
