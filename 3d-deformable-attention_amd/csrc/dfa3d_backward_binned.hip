@@ -6,7 +6,8 @@
 // scalar updates of grad_dist per sampling point.  So the points are first binned by the image tile they
 // fall in, and one workgroup per tile accumulates that tile of grad_value and grad_dist in LDS and writes it
 // out once: grad_value rows without any atomics (a lane group owns each tile row), grad_dist taps with
-// LDS atomics, which are some 25 times faster than device-memory ones.
+// plain LDS updates handed out by integer tickets (LDS floating-point atomics only for the few taps that
+// meet another one of the same pass at their address).
 //
 //   plan_and_clear_kernel       validates the level table, lays out the tiles (bins), clears counters
 //   bin_points_kernel<0>        points per bin (LDS histogram per block, one atomic per touched bin)
@@ -271,10 +272,11 @@ __global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws) {
 //            row's tasks takes the staged grad_out row, leaves the dot product for phase C and
 //            accumulates weight * grad_out in registers; the row sum is added to the LDS tile with a
 //            plain read-modify-write (nobody else touches that row during the pass)
-//   phase C  thread = point: per-point gradients from the four dots; grad_dist taps go to the LDS
-//            tile with atomics (8 scalars per point)
-// After the item's last pass the tile is flushed to memory once (atomic adds: chunks of one bin
-// and the halos of neighbouring bins overlap).
+//   phase C  thread = point: per-point gradients from the four dots; the 8 grad_dist taps of a point go
+//            to the LDS tile (first taker of an address: plain update, later ones: atomics)
+// After the item's last pass the tile is flushed to memory once: stores for the inner rows of an item that
+// holds all the points of its bin, atomic adds for the rest (the chunks of one bin overlap, and so do the
+// rims of neighbouring bins).
 // ---------------------------------------------------------------------------------------
 
 // Optional phase timing of the tile kernel (development builds only, -DDFA3D_TILE_TIMING): thread 0
