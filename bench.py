@@ -274,13 +274,20 @@ def main():
     bwd_all_ms, bwd_all_best = event_time(backward_call, a.kernel_reps, prep=zero)
     fill_ms, _ = event_time(zero, a.kernel_reps)
 
-    def entry(name, ms, best, nbytes):
+    def entry(name, ms, best, nbytes, key=None):
         gbs = nbytes / (ms * 1e-3) / 1e9
-        return {"kernel": name, "avg_ms": round(ms, 4), "min_ms": round(best, 4), "algorithmic_bytes": nbytes,
-                "achieved_gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
-                "points_per_s": w.points / (ms * 1e-3)}
+        e = {"kernel": name, "avg_ms": round(ms, 4), "min_ms": round(best, 4), "algorithmic_bytes": nbytes,
+             "achieved_gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+             "points_per_s": w.points / (ms * 1e-3)}
+        traffic = MEASURED_TRAFFIC_BYTES.get((a.workload, key)) if not bf16 else None
+        if traffic:
+            # bytes the hardware counters saw on the memory side of the L2, over the time measured here
+            e["counter_traffic_gbs"] = round(traffic / (ms * 1e-3) / 1e9, 1)
+            e["counter_traffic_frac_of_hbm_peak"] = round(traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        return e
 
-    kernels = {"forward": entry("fwd_attention_kernel (depth score + attention, one launch)", fwd_ms, fwd_best, fwd_bytes)}
+    kernels = {"forward": entry("fwd_attention_kernel (depth score + attention, one launch)", fwd_ms, fwd_best, fwd_bytes,
+                                "forward")}
     if ws_bytes:
         # binning kernels alone, then the tile kernel alone on the workspace they prepared
         _lib.set_tunable("bwd_stage", 1)
@@ -294,7 +301,8 @@ def main():
 
         tile_ms, tile_best = event_time(backward_call, a.kernel_reps, prep=prepare_tile)
         _lib.set_tunable("bwd_stage", 0)
-        kernels["backward_tile"] = entry("tile_backward_kernel (all gradients, one launch)", tile_ms, tile_best, bwd_bytes)
+        kernels["backward_tile"] = entry("tile_backward_kernel (all gradients, one launch)", tile_ms, tile_best, bwd_bytes,
+                                         "backward_tile")
         kernels["backward_binning"] = {"kernel": "plan_and_clear + bin_points<0> + bin_scan + bin_points<1> (4 launches)",
                                        "avg_ms": round(bin_ms, 4), "min_ms": round(bin_best, 4)}
         dom = "backward_tile" if tile_ms >= fwd_ms else "forward"
