@@ -451,6 +451,8 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
   const int group = wave * RPI + lane / LPR, cl = lane % LPR;
   const int passes = (C + VEC * LPR - 1) / (VEC * LPR);
   const int LP = L * P;
+  const int my_set = tid / PP, slot = tid % PP;         // the workgroup has at least 2 PP threads; halves 0 and 1
+                                                        // own alternate passes, further threads none
 
   for (int i = tid; i < R * (C + D); i += n_thr) smem[i] = 0;   // gv and gd are adjacent
   TT_DECL
@@ -481,33 +483,48 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
     const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * Md * D : nullptr, FUSED ? (size_t)S * Md * D * sizeof(T) : 0);
     const rsrc_t go_r = make_rsrc(grad_out + (size_t)b * Q * M * C, (size_t)Q * M * C * sizeof(T));
 
-    for (int base = 0; base < n_item; base += PP) {               // uniform over the workgroup
-      const int cnt_pts = min(PP, n_item - base);
-      // ---------------- phase A: one thread per point ----------------
-      for (int i = tid; i < R; i += n_thr) cnt[i] = 0;
-      const bool live = tid < cnt_pts;
-      size_t gp = 0;
+    // Per-point state of the pass a thread owns.  With twice as many threads as points per pass the two halves
+    // of the workgroup own alternate passes: while one half runs phase C of pass i, the other runs phase A of
+    // pass i + 1 (two dependent memory round trips), which then costs no time of its own.
+    // What phase C needs of a point, kept small: it stays in registers through the rows phase, where every
+    // register counts.  Complements (1 - lh, ...) are formed again where they are used.
+    uint32_t st_gp = 0;                                 // index of the point
+    float st_a = 0, sc[4], hl[4];                       // weight; corner scores; upper minus lower depth tap per corner
+    float st_lh = 0, st_lw = 0, st_ld = 0;              // fractional parts along h, w, depth
+    int st_d0 = 0;                                      // lower depth bin
+    uint32_t st_tr01 = 0xFFFFFFFFu, st_tr23 = 0xFFFFFFFFu;   // tile rows of the corners, 16 bits each, 0xFFFF = none
+    unsigned st_bits = 0;            // bit k: corner k inside the map; 4: depth inside; 5, 6: lower, upper tap exists; 7: live
+    // ---------------- phase A: one thread per point ----------------
+    auto phase_a = [&](int base, int (&tr)[4], float (&wk)[4]) {
+      for (int i = slot; i < R; i += PP) cnt[i] = 0;
+      const bool live = slot < n_item - base;
       Point2D<float> g;
       DepthTap<float> tap;
-      float a = 0, sc[4], lo[4], hi[4], wk[4];
-      int tr[4];
+      size_t gp = 0;
+      float a = 0;
+      unsigned on_bits = 0;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) { tr[k] = -1; wk[k] = 0; sc[k] = 0; lo[k] = 0; hi[k] = 0; g.key[k] = -1; }
+      for (int k = 0; k < 4; ++k) { sc[k] = 0; hl[k] = 0; g.key[k] = -1; }
       g.inside = false; g.lh = g.lw = g.hh = g.hw = 0; g.h0 = g.w0 = 0;
       tap.inside = tap.lo_ok = tap.hi_ok = false; tap.d0 = 0; tap.ld = tap.hd = 0;
       uint32_t my_goff = kNoRow;
       if (live) {
-        gp = ws.entries[seg + base + tid];
-        const float4 rec = ws.recs[seg + base + tid];
+        gp = ws.entries[seg + base + slot];
+        const float4 rec = ws.recs[seg + base + slot];
         const size_t unit = gp / LP;
         a = rec.w;
         g = locate_2d<float>(rec.x, rec.y, H, W, start);
         if (FUSED) {
           tap = locate_depth<float>(rec.z, Dd);
 #ifdef DFA3D_EXPERIMENT
-          if (diag & 32) { for (int k = 0; k < 4; ++k) { sc[k] = 0.5f; lo[k] = 0.1f; hi[k] = 0.2f; } } else   // cost of the depth taps
+          if (diag & 32) { for (int k = 0; k < 4; ++k) { sc[k] = 0.5f; hl[k] = 0.1f; } } else   // cost of the depth taps
 #endif
-          corner_scores<T, float>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
+          {
+            float lo[4], hi[4];
+            corner_scores<T, float>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) hl[k] = hi[k] - lo[k];
+          }
         } else {
           const T *si = score_in + gp * 4;
 #pragma unroll
@@ -517,6 +534,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           if (g.key[k] >= 0) {
+            on_bits |= 1u << k;
             const int ry = g.h0 + (k >= 2 ? 1 : 0) - y0, rx = g.w0 + ((k == 1 || k == 2) ? 1 : 0) - x0;
             if (ry >= 0 && ry <= TY && rx >= 0 && rx <= TX) {
               tr[k] = ry * TW + rx;
@@ -525,12 +543,142 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           }
         }
       }
-      if (tid < PP) goff[tid] = my_goff;
+      goff[slot] = my_goff;
+      st_gp = (uint32_t)gp; st_a = a; st_lh = g.lh; st_lw = g.lw; st_ld = tap.ld; st_d0 = tap.d0;
+      st_tr01 = ((uint32_t)tr[0] & 0xFFFFu) | ((uint32_t)tr[1] << 16);
+      st_tr23 = ((uint32_t)tr[2] & 0xFFFFu) | ((uint32_t)tr[3] << 16);
+      st_bits = on_bits | (tap.inside ? 16u : 0u) | (tap.lo_ok ? 32u : 0u) | (tap.hi_ok ? 64u : 0u) | (live ? 128u : 0u);
+    };
+    // The loop is rotated: a turn runs phase C of the previous pass on the half that owns it and, meanwhile,
+    // phase A of this pass on the other half; then sort and rows of this pass on everybody.  One extra turn
+    // finishes the last pass.
+    for (int pass_idx = 0;; ++pass_idx) {                        // uniform over the workgroup
+      const int base = pass_idx * PP;
+      const bool has = base < n_item;
+      const bool mine = has && my_set == (pass_idx & 1);         // this thread's half owns the pass
+      const bool prev_mine = pass_idx > 0 && my_set == ((pass_idx - 1) & 1);
+      int tr[4] = {-1, -1, -1, -1};                               // of this pass: used until its tasks are placed
+      float wk[4] = {0, 0, 0, 0};
+      if (mine) phase_a(base, tr, wk);
+
+      // ---------------- phase C: per-point gradients, grad_dist taps into the LDS tile ----------------
+      // LDS floating-point atomics retire about 0.3 lanes per clock per CU on this part, integer ones more
+      // than twenty times as many.  So every tap first swaps this pass's tag into a word that belongs to its
+      // tile address (the words live where the grad_out rows were staged: the rows phase is over).  Whoever
+      // gets something else than the tag back is the first at that address and adds at once with a plain
+      // read-modify-write: nobody else touches the address before the barrier below.  Only the others (under
+      // a fifth of the taps at 256 points per pass) use the floating-point atomic, after that barrier.  Stale
+      // words cannot do harm: one that happens to equal the tag just sends its address's taps to the atomics.
+      int *tickets = reinterpret_cast<int *>(gstage);
+      const bool ticketed = FUSED && R * D <= PP * C && !(diag & 1024);     // uniform over the workgroup
+      ++pass_tag;
+      // the previous pass's points as phase A left them
+      Point2D<float> g;
+      DepthTap<float> tap;
+      g.lh = st_lh; g.lw = st_lw; g.hh = 1 - st_lh; g.hw = 1 - st_lw;
+      tap.inside = (st_bits & 16u) != 0; tap.lo_ok = (st_bits & 32u) != 0; tap.hi_ok = (st_bits & 64u) != 0;
+      tap.d0 = st_d0; tap.ld = st_ld; tap.hd = tap.inside ? 1 - st_ld : 0.f;
+      int trc[4] = {(int)(int16_t)(st_tr01 & 0xFFFFu), (int)(int16_t)(st_tr01 >> 16),
+                    (int)(int16_t)(st_tr23 & 0xFFFFu), (int)(int16_t)(st_tr23 >> 16)};
+      const unsigned on_bits = st_bits & 15u;
+      const bool live = (st_bits & 128u) != 0;
+      const float a = st_a;
+      const size_t gp = st_gp;
+      float gs[4] = {0, 0, 0, 0};
+      unsigned first_mask = 0;              // bit 2k / 2k+1: this thread took the first ticket of corner k's lower / upper tap
+#ifdef DFA3D_EXPERIMENT
+      if (prev_mine && live && !(diag & 512)) {               // cost of phase C
+#else
+      if (prev_mine && live) {
+#endif
+        float s[4], ga = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const float dk = dots[slot * 4 + k];
+          const bool on = on_bits >> k & 1;
+          const float bk = g.bil(k);
+          gs[k] = on ? bk * a * dk : 0.f;
+          s[k] = on ? sc[k] * dk : 0.f;
+          ga += bk * s[k];
+        }
+        const float gx = (float)W * a * (g.hh * (s[1] - s[0]) + g.lh * (s[2] - s[3]));
+        const float gy = (float)H * a * (g.hw * (s[3] - s[0]) + g.lw * (s[2] - s[1]));
+        float *gl = grad_loc + gp * gl_stride;
+        if (!FUSED) { gl[0] = gx; gl[1] = gy; }
+        if (FUSED) {
+          if (grad_score_in != nullptr) {
+            const T *gi = grad_score_in + gp * 4;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) gs[k] += Elem<T>::ld(gi + k);
+          }
+          if (grad_wu != nullptr) {       // weight_update = sum over points of attn * mean corner score
+            const float gw = grad_wu[gp / LP] * 0.25f;
+            ga += gw * (sc[0] + sc[1] + sc[2] + sc[3]);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) gs[k] += gw * a;
+          }
+          float gz = 0;
+          int at8[8];                               // tile address of each of the eight taps, -1 = no tap
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const bool taps = trc[k] >= 0 && tap.inside && gs[k] != 0 && !(diag & 2);
+            const int at = trc[k] * D + tap.d0;
+            at8[2 * k] = (taps && tap.lo_ok) ? at : -1;
+            at8[2 * k + 1] = (taps && tap.hi_ok) ? at + 1 : -1;
+            if (!taps) {
+              gs[k] = ((on_bits >> k & 1) && tap.inside) ? gs[k] : 0.f;      // no taps below for this corner
+              if (!(trc[k] >= 0 && tap.inside) || (diag & 2)) trc[k] = -1;
+            }
+            gz += ((on_bits >> k & 1) && tap.inside) ? gs[k] * hl[k] : 0.f;
+          }
+          gl[0] = gx; gl[1] = gy; gl[2] = gz * (float)Dd;      // one 12-byte store
+          grad_attn[gp] = ga;                       // all stores before the tile updates: they complete slowly
+          if (ticketed) {
+            // the eight swaps back to back, then the reads of the first takers, then their writes: one LDS
+            // round trip each instead of one per tap (a thread's eight addresses are all different)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              if (at8[j] >= 0 && atomicExch(&tickets[at8[j]], pass_tag) != pass_tag) first_mask |= 1u << j;
+            float cur8[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) cur8[j] = (first_mask >> j & 1) ? gd[at8[j]] : 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              if (first_mask >> j & 1) gd[at8[j]] = cur8[j] + ((j & 1) ? tap.ld : tap.hd) * gs[j >> 1];
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              if (at8[j] >= 0) atomicAdd(gd + at8[j], ((j & 1) ? tap.ld : tap.hd) * gs[j >> 1]);
+          }
+        } else if (grad_score_out != nullptr) {
+          float *go4 = grad_score_out + gp * 4;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) go4[k] = gs[k];
+          grad_attn[gp] = ga;
+        } else {
+          grad_attn[gp] = ga;
+        }
+      }
+      if (ticketed && pass_idx > 0) {
+        __syncthreads();                                 // plain updates done before the atomic ones start
+        if (prev_mine && live) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            if (trc[k] >= 0 && gs[k] != 0) {
+              float *dst = gd + trc[k] * D + tap.d0;
+              if (tap.lo_ok && !(first_mask & (1u << (2 * k)))) atomicAdd(dst, tap.hd * gs[k]);
+              if (tap.hi_ok && !(first_mask & (2u << (2 * k)))) atomicAdd(dst + 1, tap.ld * gs[k]);
+            }
+          }
+        }
+      }
+      TT_MARK(5);
+      if (!has) break;
       __syncthreads();                                   // counters cleared, goff visible
       TT_MARK(1);
       int rank[4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) rank[k] = tr[k] >= 0 ? atomicAdd(&cnt[tr[k]], 1) : 0;
+      for (int k = 0; k < 4; ++k) rank[k] = (mine && tr[k] >= 0) ? atomicAdd(&cnt[tr[k]], 1) : 0;
       // stage the grad_out rows of this wavefront's 64 points (lanes over channels)
       for (int pass = 0; pass < passes; ++pass) {
         const int chan = (pass * LPR + cl) * VEC;
@@ -551,7 +699,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
       // Exclusive prefix of the row counters.  Every wavefront that places tasks computes it, two rows per
       // lane and 128 rows per step, and writes the same numbers: it can go on with its own copy without
       // waiting for the others.
-      if (wave * kWave < PP) {
+      if (mine) {                                        // whole wavefronts
         int run = 0;
         for (int r0 = 0; r0 < R; r0 += 2 * kWave) {
           const int r = r0 + 2 * lane;
@@ -565,14 +713,14 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
       }
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        if (tid >= PP) {
+        if (!mine) {
         } else if (tr[k] >= 0) {
           RowTask t;
           t.w = wk[k];
-          t.who = (uint32_t)(tid * 4 + k);
+          t.who = (uint32_t)(slot * 4 + k);
           tasks[offs[tr[k]] + rank[k]] = t;
         } else {
-          dots[tid * 4 + k] = 0;                         // no row will write this dot
+          dots[slot * 4 + k] = 0;                        // no row will write this dot
         }
       }
       __syncthreads();                                   // tasks grouped by row, grad_out rows staged
@@ -658,109 +806,6 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
       }
       __syncthreads();                                   // dots complete
       TT_MARK(4);
-
-      // ---------------- phase C: per-point gradients, grad_dist taps into the LDS tile ----------------
-      // LDS floating-point atomics retire about 0.3 lanes per clock per CU on this part, integer ones more
-      // than twenty times as many.  So every tap first swaps this pass's tag into a word that belongs to its
-      // tile address (the words live where the grad_out rows were staged: the rows phase is over).  Whoever
-      // gets something else than the tag back is the first at that address and adds at once with a plain
-      // read-modify-write: nobody else touches the address before the barrier below.  Only the others (under
-      // a fifth of the taps at 256 points per pass) use the floating-point atomic, after that barrier.  Stale
-      // words cannot do harm: one that happens to equal the tag just sends its address's taps to the atomics.
-      int *tickets = reinterpret_cast<int *>(gstage);
-      const bool ticketed = FUSED && R * D <= PP * C && !(diag & 1024);     // uniform over the workgroup
-      ++pass_tag;
-      float gs[4] = {0, 0, 0, 0};
-      unsigned first_mask = 0;              // bit 2k / 2k+1: this thread took the first ticket of corner k's lower / upper tap
-#ifdef DFA3D_EXPERIMENT
-      if (live && !(diag & 512)) {                       // cost of phase C
-#else
-      if (live) {
-#endif
-        float s[4], ga = 0;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const float dk = dots[tid * 4 + k];
-          const bool on = g.key[k] >= 0;
-          const float bk = g.bil(k);
-          gs[k] = on ? bk * a * dk : 0.f;
-          s[k] = on ? sc[k] * dk : 0.f;
-          ga += bk * s[k];
-        }
-        const float gx = (float)W * a * (g.hh * (s[1] - s[0]) + g.lh * (s[2] - s[3]));
-        const float gy = (float)H * a * (g.hw * (s[3] - s[0]) + g.lw * (s[2] - s[1]));
-        float *gl = grad_loc + gp * gl_stride;
-        if (!FUSED) { gl[0] = gx; gl[1] = gy; }
-        if (FUSED) {
-          if (grad_score_in != nullptr) {
-            const T *gi = grad_score_in + gp * 4;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) gs[k] += Elem<T>::ld(gi + k);
-          }
-          if (grad_wu != nullptr) {       // weight_update = sum over points of attn * mean corner score
-            const float gw = grad_wu[gp / LP] * 0.25f;
-            ga += gw * (sc[0] + sc[1] + sc[2] + sc[3]);
-#pragma unroll
-            for (int k = 0; k < 4; ++k) gs[k] += gw * a;
-          }
-          float gz = 0;
-          int at8[8];                               // tile address of each of the eight taps, -1 = no tap
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const bool taps = tr[k] >= 0 && tap.inside && gs[k] != 0 && !(diag & 2);
-            const int at = tr[k] * D + tap.d0;
-            at8[2 * k] = (taps && tap.lo_ok) ? at : -1;
-            at8[2 * k + 1] = (taps && tap.hi_ok) ? at + 1 : -1;
-            if (!taps) {
-              gs[k] = (g.key[k] >= 0 && tap.inside) ? gs[k] : 0.f;      // no taps below for this corner
-              if (!(tr[k] >= 0 && tap.inside) || (diag & 2)) tr[k] = -1;
-            }
-            gz += (g.key[k] >= 0 && tap.inside) ? gs[k] * (hi[k] - lo[k]) : 0.f;
-          }
-          gl[0] = gx; gl[1] = gy; gl[2] = gz * (float)Dd;      // one 12-byte store
-          grad_attn[gp] = ga;                       // all stores before the tile updates: they complete slowly
-          if (ticketed) {
-            // the eight swaps back to back, then the reads of the first takers, then their writes: one LDS
-            // round trip each instead of one per tap (a thread's eight addresses are all different)
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-              if (at8[j] >= 0 && atomicExch(&tickets[at8[j]], pass_tag) != pass_tag) first_mask |= 1u << j;
-            float cur8[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) cur8[j] = (first_mask >> j & 1) ? gd[at8[j]] : 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-              if (first_mask >> j & 1) gd[at8[j]] = cur8[j] + ((j & 1) ? tap.ld : tap.hd) * gs[j >> 1];
-          } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-              if (at8[j] >= 0) atomicAdd(gd + at8[j], ((j & 1) ? tap.ld : tap.hd) * gs[j >> 1]);
-          }
-        } else if (grad_score_out != nullptr) {
-          float *go4 = grad_score_out + gp * 4;
-#pragma unroll
-          for (int k = 0; k < 4; ++k) go4[k] = gs[k];
-          grad_attn[gp] = ga;
-        } else {
-          grad_attn[gp] = ga;
-        }
-      }
-      if (ticketed) {
-        __syncthreads();                                 // plain updates done before the atomic ones start
-        if (live) {
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            if (tr[k] >= 0 && gs[k] != 0) {
-              float *dst = gd + tr[k] * D + tap.d0;
-              if (tap.lo_ok && !(first_mask & (1u << (2 * k)))) atomicAdd(dst, tap.hd * gs[k]);
-              if (tap.hi_ok && !(first_mask & (2u << (2 * k)))) atomicAdd(dst + 1, tap.ld * gs[k]);
-            }
-          }
-        }
-      }
-      // no barrier here: what the next pass writes before its first barrier (row counters, grad_out offsets)
-      // was last read before this pass's later barriers
-      TT_MARK(5);
     }
     __syncthreads();                                     // the tile is complete
 
@@ -1047,6 +1092,7 @@ static TileConfig pick_tile_config(int kind, int C, int D, int tile_hint, int bl
   TileConfig c;
   c.block = kind == 2 ? 256 : (block_hint == 256 ? 256 : 512);
   c.pp = (pass_hint == 128 || pass_hint == 256) ? pass_hint : 256;
+  if (kind != 2 && c.pp * 2 > c.block) c.pp = c.block / 2;   // the fused tile kernel wants two halves of PP threads
   if (c.pp > c.block) c.pp = c.block;
   const int cand[][2] = {{16, 16}, {8, 16}, {8, 8}, {4, 8}, {4, 4}, {2, 4}, {2, 2}, {1, 1}};
   c.ty = c.tx = 1;
