@@ -32,8 +32,8 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
 # scaled by what the same counter reads for the library's plain 1 GiB streaming copy (profiles/).
 MEASURED_TRAFFIC_BYTES = {
     # profiles/fwd_attention_and_tile_backward_base_fp32.txt
-    ("base", "forward"): 5.21e9,
-    ("base", "backward_tile"): 4.31e9,
+    ("base", "forward"): 5.22e9,
+    ("base", "backward_tile"): 4.15e9,
 }
 
 
