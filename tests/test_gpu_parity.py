@@ -398,6 +398,27 @@ def test_fp32_random_shapes_two_stage_and_shared_distribution(oracle, seed):
     _compare([out.detach().cpu(), want[1], *[x.cpu() for x in grads]], [want[0], want[1], *want[3:]], F32_FWD, F32_BWD)
 
 
+@pytest.mark.parametrize("setting", [dict(block=256), dict(**{"pass": 128}), dict(tile=404), dict(tile=816),
+                                     dict(tile=203, chunk=64), dict(chunk=256), dict(vec=4), dict(vec=8, tile=404)],
+                         ids=lambda d: "-".join(f"{k}{v}" for k, v in d.items()))
+def test_launch_tunables_do_not_change_results(oracle, setting):
+    """Tile shape, workgroup size, points per pass, points per work item and channels per lane of the binned
+    backward are launch parameters only."""
+    from dfa3D import _lib
+    dev = _dev()
+    t = tiny_case(70, B=2, C=32, M=8, Q=700, P=8, D=16, levels=((37, 52), (19, 26), (7, 9)), dtype=torch.float32)
+    inp = _as_inputs(t)
+    want = _oracle_one_stage(oracle, inp)
+    try:
+        for k, v in setting.items():
+            _lib.set_tunable(k, v)
+        _compare(_gpu_one_stage(inp, dev), want, F32_FWD, F32_BWD)
+        _compare(_gpu_two_stage(inp, dev, sliced=False), want, F32_FWD, F32_BWD)
+    finally:
+        for k in setting:
+            _lib.set_tunable(k, 0)
+
+
 def test_fp32_base_shape_two_stage_matches_checker(oracle):
     from dfa3D.workloads import WORKLOADS, make_inputs
     dev = _dev()
