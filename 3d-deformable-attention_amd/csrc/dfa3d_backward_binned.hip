@@ -521,7 +521,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
 #endif
           {
             float lo[4], hi[4];
-            corner_scores<T, float>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
+            corner_scores<T, float, true>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
 #pragma unroll
             for (int k = 0; k < 4; ++k) hl[k] = hi[k] - lo[k];
           }
@@ -944,7 +944,7 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
         const Point2D<float> g = locate_2d<float>(rec.x, rec.y, H, W, start);
         tap = locate_depth<float>(rec.z, Dd);
         float sc[4], lo[4], hi[4];
-        corner_scores<T, float>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
+        corner_scores<T, float, true>(dist_r, g.key, tap, m, M, D, sc, lo, hi);
         const T *gi = grad_score + gp * 4;
         float gz = 0;
 #pragma unroll

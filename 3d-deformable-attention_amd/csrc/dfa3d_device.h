@@ -323,13 +323,26 @@ template <> struct BufPair<double> {
   }
 };
 template <> struct BufPair<__hip_bfloat16> {
-  // two 2-byte loads; corner_scores uses ld_aligned4 instead when rows are 8-byte aligned
+  // two 2-byte loads: rows of an odd number of bins
   static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, float &x, float &y) {
     x = BufElem<__hip_bfloat16>::ld(r, off);
     y = BufElem<__hip_bfloat16>::ld(r, off == kNoRow ? kNoRow : off + 2);
   }
-  // Rows that start on 8-byte boundaries (D % 4 == 0): one 8-byte load of the aligned group of four
-  // bins holds the pair unless it starts at the group's last bin (then one extra 2-byte load).
+  // One 8-byte load from the 4-byte boundary at or below the pair: it holds the pair whichever half of its
+  // first word the pair starts in.  The load may reach up to four bytes past the buffer's end; the hardware
+  // checks the range word by word, so the words inside come back and the one outside reads as zero.  Needs a
+  // buffer whose size is a multiple of 4 bytes (an even number of bins per row), or the last word could be
+  // cut in the middle and dropped.
+  static __device__ __forceinline__ void ld_word_aligned(rsrc_t r, uint32_t off, float &x, float &y) {
+    const uint32_t shift = (off & 2u) << 3;              // 0 or 16 bits into the first word
+    const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, off == kNoRow ? kNoRow : (off & ~3u), 0, 0);
+    const unsigned long long v = (((unsigned long long)t.y << 32) | t.x) >> shift;
+    x = bf16_bits_to_float((uint32_t)v & 0xFFFFu);
+    y = bf16_bits_to_float((uint32_t)(v >> 16) & 0xFFFFu);
+  }
+  // Rows that start on 8-byte boundaries (D % 4 == 0): one 8-byte load of the aligned group of four bins
+  // holds the pair unless it starts at the group's last bin (then one extra 2-byte load).  Two instructions,
+  // but every access is naturally aligned: faster where the lines are already in the L1 (the tile kernels).
   static __device__ __forceinline__ void ld_aligned4(rsrc_t r, uint32_t off, float &x, float &y) {
     const bool none = off == kNoRow;
     const uint32_t idx = (off >> 1) & 3;
@@ -341,12 +354,14 @@ template <> struct BufPair<__hip_bfloat16> {
   }
 };
 
-template <typename T> struct PairLoader {
+// LOCAL: the caller's taps mostly hit lines its workgroup has just used (tile kernels)
+template <typename T, bool LOCAL> struct PairLoader {
   static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, int, T &x, T &y) { BufPair<T>::ld(r, off, x, y); }
 };
-template <> struct PairLoader<__hip_bfloat16> {
+template <bool LOCAL> struct PairLoader<__hip_bfloat16, LOCAL> {
   static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, int D, float &x, float &y) {
-    if ((D & 3) == 0) BufPair<__hip_bfloat16>::ld_aligned4(r, off, x, y);
+    if (LOCAL && (D & 3) == 0) BufPair<__hip_bfloat16>::ld_aligned4(r, off, x, y);
+    else if ((D & 1) == 0) BufPair<__hip_bfloat16>::ld_word_aligned(r, off, x, y);
     else BufPair<__hip_bfloat16>::ld(r, off, x, y);
   }
 };
@@ -354,7 +369,7 @@ template <> struct PairLoader<__hip_bfloat16> {
 // Depth scores of the four corners of one point: linear interpolation along depth of the
 // distribution stored at each corner pixel, zero outside the map / outside [0, Dd-1].
 // `dist_r` describes batch element b of dist; lo/hi return the two taps per corner.
-template <typename T, typename A>
+template <typename T, typename A, bool LOCAL = false>
 __device__ __forceinline__ void corner_scores(rsrc_t dist_r, const int (&key)[4], const DepthTap<A> &tap, int m, int M,
                                               int D, A (&score)[4], A (&lo)[4], A (&hi)[4]) {
   if (D >= 2) {
@@ -366,7 +381,7 @@ __device__ __forceinline__ void corner_scores(rsrc_t dist_r, const int (&key)[4]
     for (int k = 0; k < 4; ++k) {
       const uint32_t row = (uint32_t)(((key[k] * M + m) * D + db) * (int)sizeof(T));
       A x, y;
-      PairLoader<T>::ld(dist_r, (key[k] >= 0 && tap.inside) ? row : kNoRow, D, x, y);
+      PairLoader<T, LOCAL>::ld(dist_r, (key[k] >= 0 && tap.inside) ? row : kNoRow, D, x, y);
       lo[k] = lo_x ? x : lo_y ? y : (A)0;
       hi[k] = hi_x ? x : hi_y ? y : (A)0;
     }
