@@ -14,6 +14,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "dfa3D", "libdfa3d_hip.so")
+# yardstick kernels for bench.py (plain copy, bare gathers, LDS atomics, XCD map): not part of the operator library
+MEASURE_SRC = os.path.join(CSRC, "measure", "dfa3d_measure.hip")
+MEASURE_LIB = os.path.join(HERE, "dfa3D", "libdfa3d_measure.so")
 SOURCES = ["dfa3d_forward.hip", "dfa3d_backward.hip", "dfa3d_backward_binned.hip", "dfa3d_rebatch.hip",
            "dfa3d_api.hip"]
 HEADERS = ["dfa3d_device.h", "dfa3d_launch.h", os.path.join("..", "..", "include", "dfa3d.h")]
@@ -46,11 +49,13 @@ def build(force=False, verbose=True):
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=5) as ex:
         list(ex.map(run, jobs))
     objs = [os.path.join(OBJ, s.replace(".hip", ".o")) for s in SOURCES]
     if force or jobs or _stale(LIB, objs):
         run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
+    if force or _stale(MEASURE_LIB, [MEASURE_SRC, os.path.join(CSRC, "measure", "dfa3d_measure.h")]):
+        run([hipcc, *FLAGS, "-shared", MEASURE_SRC, "-o", MEASURE_LIB])
     return LIB
 
 

@@ -27,23 +27,46 @@ int hip_result(hipError_t e, const char *what) {
   return fail((int)e, "%s: %s", what, hipGetErrorString(e));
 }
 
-// Process-wide launch tunables (dfa3d_set_tunable); initial values may come from the environment
-// variables DFA3D_ITERS / DFA3D_VEC.
-int env_int(const char *name, int dflt) {
-  const char *s = getenv(name);
-  return (s && *s) ? atoi(s) : dflt;
+// Launch options of one call, checked.  A NULL pointer stands for the defaults.
+int check_opts(const char *fn, const dfa3d_launch_options *o, dfa3d_launch_options *out) {
+  dfa3d_launch_options r;
+  memset(&r, 0, sizeof(r));
+  if (o != nullptr) r = *o;
+  if (r.iters < 0 || r.iters > 64) return fail(DFA3D_EINVAL, "%s: options.iters must be in [0, 64]", fn);
+  if (r.iters == 0) r.iters = 1;
+  if (r.vec != 0 && r.vec != 1 && r.vec != 2 && r.vec != 4 && r.vec != 8)
+    return fail(DFA3D_EINVAL, "%s: options.vec must be 0 (automatic), 1, 2, 4 or 8", fn);
+  const int ty = r.tile / 100, tx = r.tile % 100;
+  if (r.tile != 0 && (r.tile < 0 || ty < 1 || tx < 1 || ty > 64 || tx > 64))
+    return fail(DFA3D_EINVAL, "%s: options.tile must be 0 or ty*100+tx with 1 <= ty, tx <= 64", fn);
+  if (r.block != 0 && r.block != 256 && r.block != 512)
+    return fail(DFA3D_EINVAL, "%s: options.block must be 0, 256 or 512", fn);
+  if (r.pass != 0 && r.pass != 64 && r.pass != 128 && r.pass != 256)
+    return fail(DFA3D_EINVAL, "%s: options.pass must be 0, 64, 128 or 256", fn);
+  if (r.chunk != 0 && (r.chunk < 64 || r.chunk > (1 << 20)))   // 64 = kMinChunk of the binned backward
+    return fail(DFA3D_EINVAL, "%s: options.chunk must be 0 or in [64, 2^20]", fn);
+  if (r.reserved != 0) return fail(DFA3D_EINVAL, "%s: options.reserved must be 0", fn);
+  *out = r;
+  return 0;
 }
-std::atomic<int> g_iters{env_int("DFA3D_ITERS", 1)};
-std::atomic<int> g_vec{env_int("DFA3D_VEC", 0)};
+
+#ifdef DFA3D_EXPERIMENT
+// Development builds only: switches that cut parts out of the backward kernels to see what they cost
+// (results are then incomplete).  Not part of the library's ABI.
 std::atomic<int> g_diag{0};
-std::atomic<int> g_tile{0};
-std::atomic<int> g_block{0};
-std::atomic<int> g_chunk{0};
 std::atomic<int> g_stage{0};
-std::atomic<int> g_pass{0};
-std::atomic<int> g_binned{1};
-int tune_iters() { const int v = g_iters.load(std::memory_order_relaxed); return v < 1 ? 1 : v; }
-int tune_vec() { return g_vec.load(std::memory_order_relaxed); }
+#endif
+
+void apply_opts(dfa3d::BwdArgs &a, const dfa3d_launch_options &o) {
+  a.iters = o.iters; a.vec_hint = o.vec; a.tile_hint = o.tile; a.block_hint = o.block; a.chunk_hint = o.chunk;
+  a.pass_hint = o.pass; a.event_binned = o.event_binned;
+#ifdef DFA3D_EXPERIMENT
+  a.diag = g_diag.load(std::memory_order_relaxed);
+  a.stage = g_stage.load(std::memory_order_relaxed);
+#else
+  a.diag = 0; a.stage = 0;
+#endif
+}
 
 // Dimension checks shared by every entry point.  `width` is the per-head row length (C or D).
 int check_dims(const char *fn, int B, int S, int M, int width, int L, int Q, int P, int dtype) {
@@ -67,91 +90,28 @@ int check_dims(const char *fn, int B, int S, int M, int width, int L, int Q, int
 #define REQUIRE_PTR(fn, p) \
   if ((p) == nullptr) return fail(DFA3D_EINVAL, "%s: %s is NULL", fn, #p)
 
-// Plain streaming copy, 16 bytes per lane: the yardstick the profiler's HBM counters are scaled by.
-__global__ __launch_bounds__(256) void stream_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
-                                                          size_t n16) {
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
-    dst[i] = src[i];
-}
-
 }  // namespace
 
 extern "C" {
 
-int dfa3d_stream_copy(void *dst, const void *src, size_t bytes, void *stream) {
-  const char *fn = "dfa3d_stream_copy";
-  REQUIRE_PTR(fn, dst); REQUIRE_PTR(fn, src);
-  if (bytes == 0 || bytes % 16 != 0 || ((uintptr_t)dst | (uintptr_t)src) % 16 != 0)
-    return fail(DFA3D_EINVAL, "%s: size and both pointers must be non-zero multiples of 16 bytes", fn);
-  const size_t n16 = bytes / 16;
-  size_t blocks = (n16 + 255) / 256;
-  if (blocks > 256 * 32) blocks = 256 * 32;
-  hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                     (const uint4 *)src, (uint4 *)dst, n16);
-  return hip_result(hipGetLastError(), fn);
-}
-
 const char *dfa3d_last_error(void) { return g_err; }
-int dfa3d_abi_version(void) { return 6; }
+int dfa3d_abi_version(void) { return 7; }
 
-int dfa3d_set_tunable(const char *name, int value) {
-  if (name == nullptr) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: name is NULL");
-  if (!strcmp(name, "iters")) {
-    if (value < 1 || value > 64) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: iters must be in [1, 64]");
-    g_iters.store(value, std::memory_order_relaxed);
-    return 0;
-  }
-  if (!strcmp(name, "vec")) {
-    if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8)
-      return fail(DFA3D_EINVAL, "dfa3d_set_tunable: vec must be 0 (automatic), 1, 2, 4 or 8");
-    g_vec.store(value, std::memory_order_relaxed);
-    return 0;
-  }
-  if (!strcmp(name, "tile")) {
-    const int ty = value / 100, tx = value % 100;
-    if (value != 0 && (ty < 1 || tx < 1 || ty > 64 || tx > 64))
-      return fail(DFA3D_EINVAL, "dfa3d_set_tunable: tile must be 0 or ty*100+tx with 1 <= ty, tx <= 64");
-    g_tile.store(value, std::memory_order_relaxed);
-    return 0;
-  }
-  if (!strcmp(name, "block")) {
-    if (value != 0 && (value < 64 || value > 1024 || value % 64 != 0))
-      return fail(DFA3D_EINVAL, "dfa3d_set_tunable: block must be 0 or a multiple of 64 in [64, 1024]");
-    g_block.store(value, std::memory_order_relaxed);
-    return 0;
-  }
-  if (!strcmp(name, "chunk")) {
-    if (value != 0 && (value < 64 || value > (1 << 20)))   // 64 = kMinChunk of the binned backward
-      return fail(DFA3D_EINVAL, "dfa3d_set_tunable: chunk must be 0 or in [64, 2^20]");
-    g_chunk.store(value, std::memory_order_relaxed);
-    return 0;
-  }
-  if (!strcmp(name, "pass")) {
-    if (value != 0 && value != 128 && value != 256) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: pass must be 0, 128 or 256");
-    g_pass.store(value, std::memory_order_relaxed);
-    return 0;
-  }
-  if (!strcmp(name, "bwd_stage")) {
-    if (value < 0 || value > 2) return fail(DFA3D_EINVAL, "dfa3d_set_tunable: bwd_stage must be 0, 1 or 2");
-    g_stage.store(value, std::memory_order_relaxed);
-    return 0;
-  }
-  if (!strcmp(name, "binned")) {
-    g_binned.store(value != 0, std::memory_order_relaxed);
-    return 0;
-  }
-  if (!strcmp(name, "diag")) {
-    g_diag.store(value, std::memory_order_relaxed);
-    return 0;
-  }
-  return fail(DFA3D_EINVAL, "dfa3d_set_tunable: unknown tunable '%s'", name);
+#ifdef DFA3D_EXPERIMENT
+int dfa3d_experiment_set(const char *name, int value) {
+  if (name != nullptr && !strcmp(name, "diag")) { g_diag.store(value, std::memory_order_relaxed); return 0; }
+  if (name != nullptr && !strcmp(name, "bwd_stage")) { g_stage.store(value, std::memory_order_relaxed); return 0; }
+  return fail(DFA3D_EINVAL, "dfa3d_experiment_set: unknown switch");
 }
+#endif
 
 int dfa3d_ms_depth_score_sample_forward(const void *dist, const int64_t *shapes3, const int64_t *level_start,
                                         const void *loc3, void *score, int B, int S, int M, int D, int L, int Q, int P,
-                                        int dtype, void *stream) {
+                                        int dtype, const dfa3d_launch_options *opts, void *stream) {
   const char *fn = "dfa3d_ms_depth_score_sample_forward";
+  dfa3d_launch_options o;
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  if (int rc = check_opts(fn, opts, &o)) return rc;
   REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
   REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, score);
   dfa3d::DepthScoreArgs a{dist, shapes3, level_start, loc3, score, B, S, M, D, L, Q, P};
@@ -159,26 +119,30 @@ int dfa3d_ms_depth_score_sample_forward(const void *dist, const int64_t *shapes3
 }
 
 size_t dfa3d_ms_depth_score_sample_backward_workspace_bytes(int B, int S, int M, int D, int L, int Q, int P,
-                                                            int dtype) {
-  if (check_dims("dfa3d_ms_depth_score_sample_backward_workspace_bytes", B, S, M, D, L, Q, P, dtype)) return 0;
-  if (!g_binned.load(std::memory_order_relaxed)) return 0;
+                                                            int dtype, const dfa3d_launch_options *opts) {
+  const char *fn = "dfa3d_ms_depth_score_sample_backward_workspace_bytes";
+  dfa3d_launch_options o;
+  if (check_dims(fn, B, S, M, D, L, Q, P, dtype) || check_opts(fn, opts, &o)) return 0;
+  if (o.direct) return 0;
   dfa3d::DepthScoreBwdArgs a{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, B, S, M, D, L, Q, P};
-  return dfa3d::binned_depth_score_backward_workspace_bytes(a, dtype, g_tile.load(std::memory_order_relaxed));
+  return dfa3d::binned_depth_score_backward_workspace_bytes(a, dtype, o.tile);
 }
 
 int dfa3d_ms_depth_score_sample_backward(const void *dist, const int64_t *shapes3, const int64_t *level_start,
                                          const void *loc3, const void *grad_score, void *grad_dist, void *grad_loc3,
                                          void *workspace, size_t workspace_bytes,
-                                         int B, int S, int M, int D, int L, int Q, int P, int dtype, void *stream) {
+                                         int B, int S, int M, int D, int L, int Q, int P, int dtype,
+                                         const dfa3d_launch_options *opts, void *stream) {
   const char *fn = "dfa3d_ms_depth_score_sample_backward";
+  dfa3d_launch_options o;
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  if (int rc = check_opts(fn, opts, &o)) return rc;
   REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start); REQUIRE_PTR(fn, loc3);
   REQUIRE_PTR(fn, grad_score); REQUIRE_PTR(fn, grad_dist); REQUIRE_PTR(fn, grad_loc3);
   dfa3d::DepthScoreBwdArgs a{dist, shapes3, level_start, loc3, grad_score, grad_dist, grad_loc3, B, S, M, D, L, Q, P};
-  if (workspace != nullptr && g_binned.load(std::memory_order_relaxed)) {
-    const hipError_t e = dfa3d::launch_depth_score_backward_binned(
-        a, dtype, workspace, workspace_bytes, g_tile.load(std::memory_order_relaxed),
-        g_chunk.load(std::memory_order_relaxed), (hipStream_t)stream);
+  if (workspace != nullptr && !o.direct) {
+    const hipError_t e = dfa3d::launch_depth_score_backward_binned(a, dtype, workspace, workspace_bytes, o.tile, o.chunk,
+                                                                   o.event_binned, (hipStream_t)stream);
     if (e != hipErrorNotSupported) return hip_result(e, fn);
   }
   return hip_result(dfa3d::launch_depth_score_backward(a, dtype, (hipStream_t)stream), fn);
@@ -187,9 +151,11 @@ int dfa3d_ms_depth_score_sample_backward(const void *dist, const int64_t *shapes
 int dfa3d_wms_deform_attn_forward(const void *value, const int64_t *shapes, int shape_stride,
                                   const int64_t *level_start, const void *loc, int loc_stride, const void *attn,
                                   const void *score, void *out, int B, int S, int M, int C, int L, int Q, int P,
-                                  int dtype, void *stream) {
+                                  int dtype, const dfa3d_launch_options *opts, void *stream) {
   const char *fn = "dfa3d_wms_deform_attn_forward";
+  dfa3d_launch_options o;
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
+  if (int rc = check_opts(fn, opts, &o)) return rc;
   if (shape_stride < 2 || shape_stride > 3 || loc_stride < 2 || loc_stride > 3)
     return fail(DFA3D_EINVAL, "%s: shape_stride and loc_stride must be 2 or 3", fn);
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, shapes); REQUIRE_PTR(fn, level_start); REQUIRE_PTR(fn, loc);
@@ -198,7 +164,7 @@ int dfa3d_wms_deform_attn_forward(const void *value, const int64_t *shapes, int 
   a.value = value; a.dist = nullptr; a.shapes = shapes; a.shape_stride = shape_stride; a.level_start = level_start;
   a.loc = loc; a.loc_stride = loc_stride; a.attn = attn; a.score_in = score; a.out = out; a.score_out = nullptr;
   a.B = B; a.S = S; a.M = M; a.C = C; a.D = 1; a.L = L; a.Q = Q; a.P = P;
-  a.iters = tune_iters(); a.vec_hint = tune_vec();
+  a.iters = o.iters; a.vec_hint = o.vec;
   return hip_result(dfa3d::launch_forward(a, dtype, (hipStream_t)stream), fn);
 }
 
@@ -206,26 +172,25 @@ static dfa3d::BwdArgs wms_bwd_args(const void *value, const int64_t *shapes, int
                                    const int64_t *level_start, const void *loc, int loc_stride, const void *attn,
                                    const void *score, const void *grad_out, void *grad_value, void *grad_loc,
                                    int grad_loc_stride, void *grad_attn, void *grad_score, int B, int S, int M, int C,
-                                   int L, int Q, int P) {
+                                   int L, int Q, int P, const dfa3d_launch_options &o) {
   dfa3d::BwdArgs a{};
   a.value = value; a.dist = nullptr; a.shapes = shapes; a.shape_stride = shape_stride; a.level_start = level_start;
   a.loc = loc; a.loc_stride = loc_stride; a.attn = attn; a.score_in = score; a.grad_out = grad_out;
   a.grad_score_in = nullptr; a.grad_value = grad_value; a.grad_dist = nullptr; a.grad_loc = grad_loc;
   a.grad_loc_stride = grad_loc_stride; a.grad_attn = grad_attn; a.grad_score_out = grad_score;
   a.B = B; a.S = S; a.M = M; a.C = C; a.D = 1; a.L = L; a.Q = Q; a.P = P;
-  a.iters = tune_iters(); a.vec_hint = tune_vec(); a.diag = g_diag.load(std::memory_order_relaxed);
-  a.tile_hint = g_tile.load(std::memory_order_relaxed); a.block_hint = g_block.load(std::memory_order_relaxed);
-  a.chunk_hint = g_chunk.load(std::memory_order_relaxed);
-  a.stage = g_stage.load(std::memory_order_relaxed);
-  a.pass_hint = g_pass.load(std::memory_order_relaxed);
+  apply_opts(a, o);
   return a;
 }
 
-size_t dfa3d_wms_deform_attn_backward_workspace_bytes(int B, int S, int M, int C, int L, int Q, int P, int dtype) {
-  if (check_dims("dfa3d_wms_deform_attn_backward_workspace_bytes", B, S, M, C, L, Q, P, dtype)) return 0;
-  if (!g_binned.load(std::memory_order_relaxed)) return 0;
+size_t dfa3d_wms_deform_attn_backward_workspace_bytes(int B, int S, int M, int C, int L, int Q, int P, int dtype,
+                                                      const dfa3d_launch_options *opts) {
+  const char *fn = "dfa3d_wms_deform_attn_backward_workspace_bytes";
+  dfa3d_launch_options o;
+  if (check_dims(fn, B, S, M, C, L, Q, P, dtype) || check_opts(fn, opts, &o)) return 0;
+  if (o.direct) return 0;
   const dfa3d::BwdArgs a = wms_bwd_args(nullptr, nullptr, 2, nullptr, nullptr, 2, nullptr, nullptr, nullptr, nullptr,
-                                        nullptr, 2, nullptr, nullptr, B, S, M, C, L, Q, P);
+                                        nullptr, 2, nullptr, nullptr, B, S, M, C, L, Q, P, o);
   return dfa3d::binned_backward_workspace_bytes(a, 1, dtype);
 }
 
@@ -234,9 +199,11 @@ int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int
                                    const void *score, const void *grad_out, void *grad_value, void *grad_loc,
                                    int grad_loc_stride, void *grad_attn, void *grad_score,
                                    void *workspace, size_t workspace_bytes, int B, int S, int M, int C,
-                                   int L, int Q, int P, int dtype, void *stream) {
+                                   int L, int Q, int P, int dtype, const dfa3d_launch_options *opts, void *stream) {
   const char *fn = "dfa3d_wms_deform_attn_backward";
+  dfa3d_launch_options o;
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
+  if (int rc = check_opts(fn, opts, &o)) return rc;
   if (shape_stride < 2 || shape_stride > 3 || loc_stride < 2 || loc_stride > 3 || grad_loc_stride < 2 ||
       grad_loc_stride > 3)
     return fail(DFA3D_EINVAL, "%s: shape_stride, loc_stride and grad_loc_stride must be 2 or 3", fn);
@@ -246,8 +213,8 @@ int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int
   if (score != nullptr) REQUIRE_PTR(fn, grad_score);            // score == NULL: every score is 1, no gradient for it
   const dfa3d::BwdArgs a = wms_bwd_args(value, shapes, shape_stride, level_start, loc, loc_stride, attn, score,
                                         grad_out, grad_value, grad_loc, grad_loc_stride, grad_attn, grad_score, B, S,
-                                        M, C, L, Q, P);
-  if (workspace != nullptr && g_binned.load(std::memory_order_relaxed)) {
+                                        M, C, L, Q, P, o);
+  if (workspace != nullptr && !o.direct) {
     const hipError_t e = dfa3d::launch_backward_binned(a, dtype, workspace, workspace_bytes, (hipStream_t)stream);
     if (e != hipErrorNotSupported) return hip_result(e, fn);
   }
@@ -256,10 +223,13 @@ int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int
 
 int dfa3d_fused_forward(const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
                         const void *loc3, const void *attn, void *out, void *score, void *weight_update, int B, int S,
-                        int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype, void *stream) {
+                        int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype,
+                        const dfa3d_launch_options *opts, void *stream) {
   const char *fn = "dfa3d_fused_forward";
+  dfa3d_launch_options o;
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  if (int rc = check_opts(fn, opts, &o)) return rc;
   if (dist_heads != M && dist_heads != 1) return fail(DFA3D_EINVAL, "%s: dist_heads must be M or 1", fn);
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
   REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, out);
@@ -268,7 +238,7 @@ int dfa3d_fused_forward(const void *value, const void *dist, const int64_t *shap
   a.loc = loc3; a.loc_stride = 3; a.attn = attn; a.score_in = nullptr; a.out = out; a.score_out = score;
   a.weight_update = weight_update; a.dist_heads = dist_heads;
   a.B = B; a.S = S; a.M = M; a.C = C; a.D = D; a.L = L; a.Q = Q; a.P = P;
-  a.iters = tune_iters(); a.vec_hint = tune_vec();
+  a.iters = o.iters; a.vec_hint = o.vec;
   return hip_result(dfa3d::launch_forward(a, dtype, (hipStream_t)stream), fn);
 }
 
@@ -276,7 +246,8 @@ static dfa3d::BwdArgs fused_bwd_args(const void *value, const void *dist, const 
                                      const int64_t *level_start, const void *loc3, const void *attn,
                                      const void *grad_out, const void *grad_score_in, const void *grad_weight_update,
                                      void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn, int B, int S,
-                                     int M, int C, int D, int L, int Q, int P, int dist_heads) {
+                                     int M, int C, int D, int L, int Q, int P, int dist_heads,
+                                     const dfa3d_launch_options &o) {
   dfa3d::BwdArgs a{};
   a.value = value; a.dist = dist; a.shapes = shapes3; a.shape_stride = 3; a.level_start = level_start;
   a.loc = loc3; a.loc_stride = 3; a.attn = attn; a.score_in = nullptr; a.grad_out = grad_out;
@@ -284,22 +255,21 @@ static dfa3d::BwdArgs fused_bwd_args(const void *value, const void *dist, const 
   a.grad_loc_stride = 3; a.grad_attn = grad_attn; a.grad_score_out = nullptr;
   a.grad_weight_update = grad_weight_update; a.dist_heads = dist_heads;
   a.B = B; a.S = S; a.M = M; a.C = C; a.D = D; a.L = L; a.Q = Q; a.P = P;
-  a.iters = tune_iters(); a.vec_hint = tune_vec(); a.diag = g_diag.load(std::memory_order_relaxed);
-  a.tile_hint = g_tile.load(std::memory_order_relaxed); a.block_hint = g_block.load(std::memory_order_relaxed);
-  a.chunk_hint = g_chunk.load(std::memory_order_relaxed);
-  a.stage = g_stage.load(std::memory_order_relaxed);
-  a.pass_hint = g_pass.load(std::memory_order_relaxed);
+  apply_opts(a, o);
   return a;
 }
 
 size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads,
-                                            int dtype) {
-  if (check_dims("dfa3d_fused_backward_workspace_bytes", B, S, M, C, L, Q, P, dtype)) return 0;
-  if (check_dims("dfa3d_fused_backward_workspace_bytes", B, S, M, D, L, Q, P, dtype)) return 0;
-  if (!g_binned.load(std::memory_order_relaxed)) return 0;
+                                            int dtype, const dfa3d_launch_options *opts) {
+  const char *fn = "dfa3d_fused_backward_workspace_bytes";
+  dfa3d_launch_options o;
+  if (check_dims(fn, B, S, M, C, L, Q, P, dtype) || check_dims(fn, B, S, M, D, L, Q, P, dtype) ||
+      check_opts(fn, opts, &o))
+    return 0;
+  if (o.direct) return 0;
   const dfa3d::BwdArgs a = fused_bwd_args(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
                                           nullptr, nullptr, nullptr, nullptr, nullptr, B, S, M, C, D, L, Q, P,
-                                          dist_heads == 1 ? 1 : M);
+                                          dist_heads == 1 ? 1 : M, o);
   return dfa3d::binned_backward_workspace_bytes(a, 0, dtype);
 }
 
@@ -307,18 +277,21 @@ int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *sha
                          const void *loc3, const void *attn, const void *grad_out, const void *grad_score_in,
                          const void *grad_weight_update, void *grad_value, void *grad_dist, void *grad_loc3,
                          void *grad_attn, void *workspace, size_t workspace_bytes, int B, int S, int M,
-                         int C, int D, int L, int Q, int P, int dist_heads, int dtype, void *stream) {
+                         int C, int D, int L, int Q, int P, int dist_heads, int dtype,
+                         const dfa3d_launch_options *opts, void *stream) {
   const char *fn = "dfa3d_fused_backward";
+  dfa3d_launch_options o;
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  if (int rc = check_opts(fn, opts, &o)) return rc;
   if (dist_heads != M && dist_heads != 1) return fail(DFA3D_EINVAL, "%s: dist_heads must be M or 1", fn);
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
   REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
   REQUIRE_PTR(fn, grad_dist); REQUIRE_PTR(fn, grad_loc3); REQUIRE_PTR(fn, grad_attn);
   const dfa3d::BwdArgs a = fused_bwd_args(value, dist, shapes3, level_start, loc3, attn, grad_out, grad_score_in,
                                           grad_weight_update, grad_value, grad_dist, grad_loc3, grad_attn, B, S, M, C,
-                                          D, L, Q, P, dist_heads);
-  if (workspace != nullptr && g_binned.load(std::memory_order_relaxed)) {
+                                          D, L, Q, P, dist_heads, o);
+  if (workspace != nullptr && !o.direct) {
     const hipError_t e = dfa3d::launch_backward_binned(a, dtype, workspace, workspace_bytes, (hipStream_t)stream);
     if (e != hipErrorNotSupported) return hip_result(e, fn);
   }

@@ -146,10 +146,10 @@ __global__ __launch_bounds__(kBlock) void bwd_attention_kernel(
   A *gdist_b = FUSED ? grad_dist + (size_t)b * S * Md * D : nullptr;
   const int md = Md == 1 ? 0 : m;
   const rsrc_t value_r = make_rsrc(value + (size_t)b * S * M * C, (size_t)S * M * C * sizeof(T));
-  const rsrc_t gvalue_r = make_rsrc(gvalue_b, (diag & 1) ? 0 : (size_t)S * M * C * sizeof(A));
+  const rsrc_t gvalue_r = make_rsrc(gvalue_b, DFA3D_DIAG(diag, 1) ? 0 : (size_t)S * M * C * sizeof(A));
   const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * Md * D : nullptr,
                                   FUSED ? (size_t)S * Md * D * sizeof(T) : 0);
-  const rsrc_t gdist_r = make_rsrc(gdist_b, (FUSED && !(diag & 2)) ? (size_t)S * Md * D * sizeof(A) : 0);
+  const rsrc_t gdist_r = make_rsrc(gdist_b, (FUSED && !DFA3D_DIAG(diag, 2)) ? (size_t)S * Md * D * sizeof(A) : 0);
   const int q_per_iter = kWavesPerBlock * ws.upw;
 
   for (int it = 0; it < iters; ++it) {

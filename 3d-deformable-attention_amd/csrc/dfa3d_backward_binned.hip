@@ -25,6 +25,10 @@
 // A point belongs to the tile that holds its clamped base pixel (clamp(h0,0,H-1), clamp(w0,0,W-1)).
 // Semantics are those of bwd_attention_kernel (see dfa3d_backward.hip for the formulas and the
 // reference lines they restate).
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "dfa3d_device.h"
 #include "dfa3d_launch.h"
 
@@ -201,8 +205,8 @@ __global__ __launch_bounds__(256) void bin_points_kernel(
       }
       if (bin >= 0) {
         const int slot = use_lds ? s_hist[nb + bin] + atomicAdd(&s_hist[bin], 1) : atomicAdd(&gcursor[bin], 1);
-        if (!(diag & 128)) ws.entries[slot] = (uint32_t)gp;
-        if (!(diag & 64))
+        if (!DFA3D_DIAG(diag, 128)) ws.entries[slot] = (uint32_t)gp;
+        if (!DFA3D_DIAG(diag, 64))
           ws.recs[slot] = make_float4(loc[gp * loc_stride], loc[gp * loc_stride + 1],
                                       loc_stride > 2 ? loc[gp * loc_stride + 2] : 0.f, attn != nullptr ? attn[gp] : 0.f);
       }
@@ -301,7 +305,7 @@ __host__ __device__ inline TileLds tile_lds_layout(int ty, int tx, int C, int D,
   o.gv = 0;
   o.gd = o.gv + R * C;
   o.gstage = (o.gd + R * D + 3) & ~3;              // 16-byte aligned rows
-  o.tasks = (o.gstage + PP * C + 1) & ~1;          // 8-byte records
+  o.tasks = (o.gstage + (PP + 1) * C + 1) & ~1;    // PP staged rows and one row of zeros; 8-byte records
   o.dots = o.tasks + PP * 4 * 2;
   o.cnt = o.dots + PP * 4 + kWave;                 // + one scrap word per lane
   o.offs = o.cnt + R;
@@ -455,6 +459,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
                                                         // own alternate passes, further threads none
 
   for (int i = tid; i < R * (C + D); i += n_thr) smem[i] = 0;   // gv and gd are adjacent
+  for (int i = tid; i < C; i += n_thr) gstage[PP * C + i] = 0;  // the row that idle lanes of the rows phase read
   TT_DECL
 
   ItemFetch fetch;
@@ -516,9 +521,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         g = locate_2d<float>(rec.x, rec.y, H, W, start);
         if (FUSED) {
           tap = locate_depth<float>(rec.z, Dd);
-#ifdef DFA3D_EXPERIMENT
-          if (diag & 32) { for (int k = 0; k < 4; ++k) { sc[k] = 0.5f; hl[k] = 0.1f; } } else   // cost of the depth taps
-#endif
+          if (DFA3D_DIAG(diag, 32)) { for (int k = 0; k < 4; ++k) { sc[k] = 0.5f; hl[k] = 0.1f; } } else   // cost of the depth taps
           {
             float lo[4], hi[4];
             corner_scores<T, float, true>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
@@ -570,7 +573,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
       // a fifth of the taps at 256 points per pass) use the floating-point atomic, after that barrier.  Stale
       // words cannot do harm: one that happens to equal the tag just sends its address's taps to the atomics.
       int *tickets = reinterpret_cast<int *>(gstage);
-      const bool ticketed = FUSED && R * D <= PP * C && !(diag & 1024);     // uniform over the workgroup
+      const bool ticketed = FUSED && R * D <= PP * C && !DFA3D_DIAG(diag, 1024);     // uniform over the workgroup
       ++pass_tag;
       // the previous pass's points as phase A left them
       Point2D<float> g;
@@ -586,11 +589,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
       const size_t gp = st_gp;
       float gs[4] = {0, 0, 0, 0};
       unsigned first_mask = 0;              // bit 2k / 2k+1: this thread took the first ticket of corner k's lower / upper tap
-#ifdef DFA3D_EXPERIMENT
-      if (prev_mine && live && !(diag & 512)) {               // cost of phase C
-#else
-      if (prev_mine && live) {
-#endif
+      if (prev_mine && live && !DFA3D_DIAG(diag, 512)) {               // (development builds: cost of phase C)
         float s[4], ga = 0;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -621,13 +620,13 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           int at8[8];                               // tile address of each of the eight taps, -1 = no tap
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
-            const bool taps = trc[k] >= 0 && tap.inside && gs[k] != 0 && !(diag & 2);
+            const bool taps = trc[k] >= 0 && tap.inside && gs[k] != 0 && !DFA3D_DIAG(diag, 2);
             const int at = trc[k] * D + tap.d0;
             at8[2 * k] = (taps && tap.lo_ok) ? at : -1;
             at8[2 * k + 1] = (taps && tap.hi_ok) ? at + 1 : -1;
             if (!taps) {
               gs[k] = ((on_bits >> k & 1) && tap.inside) ? gs[k] : 0.f;      // no taps below for this corner
-              if (!(trc[k] >= 0 && tap.inside) || (diag & 2)) trc[k] = -1;
+              if (!(trc[k] >= 0 && tap.inside) || DFA3D_DIAG(diag, 2)) trc[k] = -1;
             }
             gz += ((on_bits >> k & 1) && tap.inside) ? gs[k] * hl[k] : 0.f;
           }
@@ -687,9 +686,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         for (int j = 0; j < stage_per_wave; j += RPI) {
           const int slot = wave * stage_per_wave + j + lane / LPR;
           float gg[VEC];
-#ifdef DFA3D_EXPERIMENT
-          if (diag & 256) { for (int i = 0; i < VEC; ++i) gg[i] = 1.f; } else   // cost of the grad_out loads
-#endif
+          if (DFA3D_DIAG(diag, 256)) { for (int i = 0; i < VEC; ++i) gg[i] = 1.f; } else   // cost of the grad_out loads
           RowVec<T, float, VEC>::ld(go_r, goff[slot] + chan_off, gg);
           if (chan < C) LdsVec<VEC>::st(gstage + slot * C + chan, gg);
         }
@@ -735,7 +732,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         {
           const int r = group;
           const int y = y0 + r / TW, x = x0 + r % TW;
-          const bool ld_ok = r < R && offs[min(r, R - 1) + 1] > offs[min(r, R - 1)] && y < H && x < W && !(diag & 8);
+          const bool ld_ok = r < R && offs[min(r, R - 1) + 1] > offs[min(r, R - 1)] && y < H && x < W && !DFA3D_DIAG(diag, 8);
           RowVec<T, float, VEC>::ld(value_r, (ld_ok ? (uint32_t)(((start + y * W + x) * M + m) * C * (int)sizeof(T)) : kNoRow) + chan_off, v_next);
         }
         for (int r0 = 0; r0 < R; r0 += kGroups) {        // uniform over the workgroup
@@ -754,12 +751,10 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           {                                              // value row of this group's next round
             const int rn = r + kGroups;
             const int yn = y0 + rn / TW, xn = x0 + rn % TW;
-            const bool ld_ok = rn < R && offs[min(rn, R - 1) + 1] > offs[min(rn, R - 1)] && yn < H && xn < W && !(diag & 8);
+            const bool ld_ok = rn < R && offs[min(rn, R - 1) + 1] > offs[min(rn, R - 1)] && yn < H && xn < W && !DFA3D_DIAG(diag, 8);
             RowVec<T, float, VEC>::ld(value_r, (ld_ok ? (uint32_t)(((start + yn * W + xn) * M + m) * C * (int)sizeof(T)) : kNoRow) + chan_off, v_next);
           }
-#ifdef DFA3D_EXPERIMENT
-          if (diag & 16) n_max = 0;                      // cost of the task loop
-#endif
+          if (DFA3D_DIAG(diag, 16)) n_max = 0;                      // cost of the task loop
           if (n_max == 0) continue;                      // wave-uniform
           // tasks in flight per group: registers decide (measured: 4 with four channels per lane, 1 with eight;
           // one more costs 1 % .. 10 % of the kernel's time)
@@ -771,8 +766,16 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           for (int t0 = 0; t0 < n_max; t0 += UT) {
             RowTask tk[UT];
             float gg[UT][VEC], part[UT];
+            // A group whose list is shorter than the wavefront's longest one idles on a task of weight zero that
+            // points at the row of zeros: nothing another point staged (a non-finite gradient, say) and no
+            // stale word is ever multiplied in.
 #pragma unroll
-            for (int j = 0; j < UT; ++j) tk[j] = row_tasks[min(t0 + j, last_task)];
+            for (int j = 0; j < UT; ++j) {
+              const RowTask t = row_tasks[min(t0 + j, last_task)];
+              const bool on = t0 + j < n_r;
+              tk[j].w = on ? t.w : 0.f;
+              tk[j].who = on ? t.who : (uint32_t)(PP * 4);
+            }
 #pragma unroll
             for (int j = 0; j < UT; ++j) lds_ld<VEC>(g_lane + (tk[j].who >> 2) * C, gg[j]);
 #pragma unroll
@@ -785,16 +788,14 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
             for (int j = 0; j < UT; ++j) part[j] = row_sum_f<LPR>(part[j]);
 #pragma unroll
             for (int j = 0; j < UT; ++j) {
-              const bool on = t0 + j < n_r;
-              const float w = on ? tk[j].w : 0.f;
 #pragma unroll
-              for (int i = 0; i < VEC; ++i) acc[i] += w * gg[j][i];
-              const int di = (on && cl == 0) ? (int)tk[j].who : dummy;
+              for (int i = 0; i < VEC; ++i) acc[i] += tk[j].w * gg[j][i];
+              const int di = cl == 0 ? (int)tk[j].who : dummy;     // an idle task's dot lands in the scrap words
               if (pass == 0) dots[di] = part[j];          // uniform branch
               else dots[di] += part[j];
             }
           }
-          if (pix_ok && chan_ok && !(diag & 1)) {
+          if (pix_ok && chan_ok && !DFA3D_DIAG(diag, 1)) {
             float *dst = gv + r * C + chan;
             float cur[VEC];
             LdsVec<VEC>::ld(dst, cur);
@@ -830,7 +831,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         if (nz) *reinterpret_cast<float4 *>(gv + r * C + c) = make_float4(0, 0, 0, 0);
         const int ry = r / TW, rx = r - ry * TW;
         const int y = y0 + ry, x = x0 + rx;
-        if (y < H && x < W && !(diag & 4)) {
+        if (y < H && x < W && !DFA3D_DIAG(diag, 4)) {
           const uint32_t off = (uint32_t)((((start + y * W + x) * M + m) * C + c) * 4);
           if (sole && ry >= 1 && ry < TY && rx >= 1 && rx < TX) {
             *reinterpret_cast<float4 *>(gvalue_b + (off >> 2)) = val;          // zeros too: full lines
@@ -849,7 +850,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         if (nz) *reinterpret_cast<float4 *>(gd + r * D + d) = make_float4(0, 0, 0, 0);
         const int ry = r / TW, rx = r - ry * TW;
         const int y = y0 + ry, x = x0 + rx;
-        if (y < H && x < W && !(diag & 4)) {
+        if (y < H && x < W && !DFA3D_DIAG(diag, 4)) {
           const uint32_t off = (uint32_t)((((start + y * W + x) * Mg + mg) * D + d) * 4);
           if (sole_d && ry >= 1 && ry < TY && rx >= 1 && rx < TX) {
             *reinterpret_cast<float4 *>(gdist_b + (off >> 2)) = val;
@@ -869,7 +870,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const int r = i / C, c = i - r * C;
         const int ry = r / TW, rx = r % TW;
         const int y = y0 + ry, x = x0 + rx;
-        if (y < H && x < W && !(diag & 4)) scatter_add(gvalue_r, gvalue_b, (uint32_t)((((start + y * W + x) * M + m) * C + c) * 4), val);
+        if (y < H && x < W && !DFA3D_DIAG(diag, 4)) scatter_add(gvalue_r, gvalue_b, (uint32_t)((((start + y * W + x) * M + m) * C + c) * 4), val);
       }
     }
     for (int i = tid; i < R * D; i += n_thr) {
@@ -879,7 +880,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const int r = i / D, d = i - r * D;
         const int ry = r / TW, rx = r % TW;
         const int y = y0 + ry, x = x0 + rx;
-        if (y < H && x < W && !(diag & 4)) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * Mg + mg) * D + d) * 4), val);
+        if (y < H && x < W && !DFA3D_DIAG(diag, 4)) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * Mg + mg) * D + d) * 4), val);
       }
     }
     }
@@ -1086,25 +1087,46 @@ static size_t tile_lds_bytes(int kind, int ty, int tx, int C, int D, int pp) {
   return (size_t)tile_lds_layout(ty, tx, C, kind == 1 ? 0 : D, pp).total * 4;
 }
 
-// Defaults: 512 threads taking 256 points per pass, and the largest tile whose LDS block still
-// lets two workgroups share a CU.
+// Defaults: 512 threads, and the largest points-per-pass and tile whose LDS block still lets two workgroups
+// share a CU.  The staged grad_out rows take pp * C floats, so long rows first shorten the pass (256 -> 128 -> 64
+// points) and only then shrink the tile below 4 x 4 pixels.
 static TileConfig pick_tile_config(int kind, int C, int D, int tile_hint, int block_hint, int pass_hint) {
   TileConfig c;
   c.block = kind == 2 ? 256 : (block_hint == 256 ? 256 : 512);
-  c.pp = (pass_hint == 128 || pass_hint == 256) ? pass_hint : 256;
-  if (kind != 2 && c.pp * 2 > c.block) c.pp = c.block / 2;   // the fused tile kernel wants two halves of PP threads
-  if (c.pp > c.block) c.pp = c.block;
+  const int pp_max = kind == 2 ? c.block : c.block / 2;      // the fused tile kernel wants two halves of pp threads
+  auto clamp_pp = [&](int pp) { return pp > pp_max ? pp_max : pp; };
   const int cand[][2] = {{16, 16}, {8, 16}, {8, 8}, {4, 8}, {4, 4}, {2, 4}, {2, 2}, {1, 1}};
-  c.ty = c.tx = 1;
+  const size_t budget = kind == 2 ? 40 * 1024 : 79 * 1024;
   const int hy = tile_hint / 100, hx = tile_hint % 100;
-  if (tile_hint > 0 && hy >= 1 && hx >= 1 && hy <= 64 && hx <= 64) {
-    c.ty = hy; c.tx = hx;
-  } else {
-    const size_t budget = kind == 2 ? 40 * 1024 : 79 * 1024;
-    for (auto &t : cand) {
-      c.ty = t[0]; c.tx = t[1];
+  const bool tile_given = tile_hint > 0 && hy >= 1 && hx >= 1 && hy <= 64 && hx <= 64;
+  const bool pass_given = pass_hint == 64 || pass_hint == 128 || pass_hint == 256;
+  c.ty = c.tx = 1;
+  c.pp = clamp_pp(pass_given ? pass_hint : 256);
+  if (tile_given) { c.ty = hy; c.tx = hx; }
+  if (tile_given && pass_given) {
+  } else if (tile_given) {
+    for (int pp : {256, 128, 64}) {
+      c.pp = clamp_pp(pp);
       if (tile_lds_bytes(kind, c.ty, c.tx, C, D, c.pp) <= budget) break;
     }
+  } else {
+    bool found = false;
+    // tiles of at least 4 x 4 pixels with the longest pass that fits; then smaller tiles with the shortest
+    for (int round = 0; round < 2 && !found; ++round) {
+      for (int pp : {256, 128, 64}) {
+        if (pass_given && pp != pass_hint) continue;
+        if (!pass_given && round == 1 && pp != 64) continue;
+        for (auto &t : cand) {
+          if ((round == 0) != (t[0] * t[1] >= 16)) continue;
+          if (tile_lds_bytes(kind, t[0], t[1], C, D, clamp_pp(pp)) <= budget) {
+            c.ty = t[0]; c.tx = t[1]; c.pp = clamp_pp(pp); found = true;
+            break;
+          }
+        }
+        if (found) break;
+      }
+    }
+    if (!found) { c.ty = c.tx = 1; c.pp = clamp_pp(pass_given ? pass_hint : 64); }
   }
   c.lds = tile_lds_bytes(kind, c.ty, c.tx, C, D, c.pp);
   return c;
@@ -1127,10 +1149,30 @@ static size_t workspace_bytes_for(const BwdArgs &a, int kind, int dtype) {
 // kind as in tile_lds_bytes; `a.dist != nullptr` is not consulted here, so dimension-only queries work
 size_t binned_backward_workspace_bytes(const BwdArgs &a, int kind, int dtype) { return workspace_bytes_for(a, kind, dtype); }
 
+// Per-device facts and per-kernel attributes are looked up once and remembered (a launch then costs no
+// runtime queries).
+static std::mutex g_launch_mutex;
+static int g_cu_count[64];                                           // 0 = not asked yet
+static std::map<std::pair<const void *, int>, size_t> g_lds_allowed;  // (kernel, device) -> dynamic LDS bytes granted
+
+static int current_device() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  return dev;
+}
+
 static int tile_grid(size_t lds, int block) {
-  int dev = 0, cus = 256;
-  if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-    cus = 256;
+  const int dev = current_device();
+  int cus;
+  {
+    std::lock_guard<std::mutex> lock(g_launch_mutex);
+    if (g_cu_count[dev] == 0) {
+      int n = 0;
+      if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+      g_cu_count[dev] = n;
+    }
+    cus = g_cu_count[dev];
+  }
   const size_t per_cu = lds > 0 ? (160 * 1024) / lds : 8;
   int wg_per_cu = (int)(per_cu < 1 ? 1 : per_cu > 8 ? 8 : per_cu);
   const int by_waves = 32 / (block / kWave);
@@ -1140,7 +1182,14 @@ static int tile_grid(size_t lds, int block) {
 
 template <typename K> static hipError_t allow_lds(K kern, size_t lds) {
   if (lds <= 64 * 1024) return hipSuccess;
-  return hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  const void *fn = reinterpret_cast<const void *>(kern);
+  const std::pair<const void *, int> key(fn, current_device());
+  std::lock_guard<std::mutex> lock(g_launch_mutex);
+  auto it = g_lds_allowed.find(key);
+  if (it != g_lds_allowed.end() && it->second >= lds) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e == hipSuccess) g_lds_allowed[key] = lds;
+  return e;
 }
 
 template <typename T, int VEC, int LPR>
@@ -1239,6 +1288,9 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
   if (a.stage == 0 || a.stage == 1) {
     if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, stream)) return e;
   }
+  if (a.event_binned != nullptr) {
+    if (hipError_t e = hipEventRecord((hipEvent_t)a.event_binned, stream)) return e;
+  }
   if (a.stage == 1) return hipSuccess;
   const size_t head_floats = (size_t)a.B * a.S * a.M * a.D;
   if (gd_heads != nullptr)       // a kernel, not a memset node: callers may capture this stream in a graph
@@ -1260,7 +1312,8 @@ size_t binned_depth_score_backward_workspace_bytes(const DepthScoreBwdArgs &d, i
 }
 
 hipError_t launch_depth_score_backward_binned(const DepthScoreBwdArgs &d, int dtype, void *workspace,
-                                              size_t workspace_bytes, int tile_hint, int chunk_hint, hipStream_t stream) {
+                                              size_t workspace_bytes, int tile_hint, int chunk_hint,
+                                              void *event_binned, hipStream_t stream) {
   if (dtype == DFA3D_F64) return hipErrorNotSupported;
   BwdArgs a{};
   a.B = d.B; a.S = d.S; a.M = d.M; a.C = 0; a.D = d.D; a.L = d.L; a.Q = d.Q; a.P = d.P;
@@ -1273,7 +1326,13 @@ hipError_t launch_depth_score_backward_binned(const DepthScoreBwdArgs &d, int dt
   const TileConfig cfg = tile_config_of(a, 2);
   const BinWorkspace ws = carve_workspace(workspace, bin_layout(a, cfg.ty, cfg.tx));
   if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, stream)) return e;
+  if (event_binned != nullptr) {
+    if (hipError_t e = hipEventRecord((hipEvent_t)event_binned, stream)) return e;
+  }
   const int grid = tile_grid(cfg.lds, cfg.block);
+  if (hipError_t e = dtype == DFA3D_F32 ? allow_lds(tile_depth_backward_kernel<float>, cfg.lds)
+                                        : allow_lds(tile_depth_backward_kernel<__hip_bfloat16>, cfg.lds))
+    return e;
   if (dtype == DFA3D_F32) {
     hipLaunchKernelGGL(tile_depth_backward_kernel<float>, dim3(grid), dim3(cfg.block), cfg.lds, stream, ws,
                        (const float *)d.dist, (const float *)d.grad_score, (float *)d.grad_dist, (float *)d.grad_loc3,

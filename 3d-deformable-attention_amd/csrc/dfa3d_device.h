@@ -24,6 +24,14 @@
 
 namespace dfa3d {
 
+// Development builds (-DDFA3D_EXPERIMENT) can cut parts out of the backward kernels to see what they cost;
+// in the library as shipped the switches are constant zero and the compiler drops them.
+#ifdef DFA3D_EXPERIMENT
+#define DFA3D_DIAG(diag, bits) (((diag) & (bits)) != 0)
+#else
+#define DFA3D_DIAG(diag, bits) false
+#endif
+
 constexpr int kWave = 64;
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = kWave * kWavesPerBlock;

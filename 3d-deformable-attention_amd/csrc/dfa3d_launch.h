@@ -68,12 +68,13 @@ struct BwdArgs {
   int B, S, M, C, D, L, Q, P;
   int iters;
   int vec_hint;
-  int diag;                          // measurement aid: bit 0 drops the grad_value updates, bit 1 the grad_dist updates
+  int diag;                          // development builds (-DDFA3D_EXPERIMENT) only, otherwise 0: parts of the kernels cut out
   int tile_hint;                     // binned path: tile edge as ty * 100 + tx (0 = automatic)
-  int block_hint;                    // binned path: threads per tile workgroup (0 = 256)
+  int block_hint;                    // binned path: threads per tile workgroup (0 = 512)
   int chunk_hint;                    // binned path: points of a bin per work item (0 = 4096)
-  int pass_hint;                     // binned path: points per pass, 128 or 256 (0 = 256)
-  int stage;                         // binned path, measurement aid: 0 all kernels, 1 binning only, 2 tile kernel only
+  int pass_hint;                     // binned path: points per pass, 64, 128 or 256 (0 = automatic)
+  int stage;                         // development builds only, otherwise 0: 1 binning kernels only, 2 tile kernel only
+  void *event_binned;                // hipEvent_t recorded between the binning kernels and the tile kernel, or nullptr
 };
 
 struct DepthScoreBwdArgs {
@@ -93,7 +94,8 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
                                   hipStream_t stream);
 size_t binned_depth_score_backward_workspace_bytes(const DepthScoreBwdArgs &d, int dtype, int tile_hint);
 hipError_t launch_depth_score_backward_binned(const DepthScoreBwdArgs &d, int dtype, void *workspace,
-                                              size_t workspace_bytes, int tile_hint, int chunk_hint, hipStream_t stream);
+                                              size_t workspace_bytes, int tile_hint, int chunk_hint,
+                                              void *event_binned, hipStream_t stream);
 
 // Camera re-batching (dfa3d_rebatch.hip); strides in elements.
 hipError_t launch_rebatch_gather(const void *src, long long cam_stride, long long batch_stride, const int *index,

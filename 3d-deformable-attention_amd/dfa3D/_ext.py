@@ -97,7 +97,8 @@ def ms_depth_score_sample_forward(value, value_spatial_shapes, value_level_start
     with torch.cuda.device(dev):
         rc = _lib.lib().dfa3d_ms_depth_score_sample_forward(
             _lib.ptr(value), _lib.ptr(value_spatial_shapes), _lib.ptr(value_level_start_index),
-            _lib.ptr(sampling_locations), _lib.ptr(score), B, S, M, D, L, Q, P, code, _lib.stream_of(value))
+            _lib.ptr(sampling_locations), _lib.ptr(score), B, S, M, D, L, Q, P, code,
+            _lib.options(), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_ms_depth_score_sample_forward")
     return score
 
@@ -124,13 +125,13 @@ def ms_depth_score_sample_backward(value, value_spatial_shapes, value_level_star
     if grad_output.numel() == 0:
         return
     code = _lib.dtype_code(value)
-    ws_bytes = _lib.lib().dfa3d_ms_depth_score_sample_backward_workspace_bytes(B, S, M, D, L, Q, P, code)
+    ws_bytes = _lib.lib().dfa3d_ms_depth_score_sample_backward_workspace_bytes(B, S, M, D, L, Q, P, code, _lib.options())
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
     with torch.cuda.device(dev):
         rc = _lib.lib().dfa3d_ms_depth_score_sample_backward(
             _lib.ptr(value), _lib.ptr(value_spatial_shapes), _lib.ptr(value_level_start_index),
             _lib.ptr(sampling_locations), _lib.ptr(grad_output), _lib.ptr(grad_value), _lib.ptr(grad_sampling_loc),
-            _lib.ptr(workspace), ws_bytes, B, S, M, D, L, Q, P, code, _lib.stream_of(value))
+            _lib.ptr(workspace), ws_bytes, B, S, M, D, L, Q, P, code, _lib.options(), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_ms_depth_score_sample_backward")
 
 
@@ -172,7 +173,7 @@ def wms_deform_attn_forward(value, value_spatial_shapes, value_level_start_index
         rc = _lib.lib().dfa3d_wms_deform_attn_forward(
             _lib.ptr(value), _lib.ptr(value_spatial_shapes), sw, _lib.ptr(value_level_start_index),
             _lib.ptr(sampling_locations), lw, _lib.ptr(attention_weights), _lib.ptr(depth_scores), _lib.ptr(out),
-            B, S, M, C, L, Q, P, _lib.dtype_code(value), _lib.stream_of(value))
+            B, S, M, C, L, Q, P, _lib.dtype_code(value), _lib.options(), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_wms_deform_attn_forward")
     return out
 
@@ -207,14 +208,15 @@ def wms_deform_attn_backward(value, value_spatial_shapes, value_level_start_inde
     if grad_output.numel() == 0:
         return
     code = _lib.dtype_code(value)
-    ws_bytes = _lib.lib().dfa3d_wms_deform_attn_backward_workspace_bytes(B, S, M, C, L, Q, P, code)
+    ws_bytes = _lib.lib().dfa3d_wms_deform_attn_backward_workspace_bytes(B, S, M, C, L, Q, P, code, _lib.options())
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
     with torch.cuda.device(dev):
         rc = _lib.lib().dfa3d_wms_deform_attn_backward(
             _lib.ptr(value), _lib.ptr(value_spatial_shapes), sw, _lib.ptr(value_level_start_index),
             _lib.ptr(sampling_locations), lw, _lib.ptr(attention_weights), _lib.ptr(depth_scores),
             _lib.ptr(grad_output), _lib.ptr(grad_value), _lib.ptr(grad_sampling_loc), gw, _lib.ptr(grad_attn_weight),
-            _lib.ptr(grad_depth_score), _lib.ptr(workspace), ws_bytes, B, S, M, C, L, Q, P, code, _lib.stream_of(value))
+            _lib.ptr(grad_depth_score), _lib.ptr(workspace), ws_bytes, B, S, M, C, L, Q, P, code, _lib.options(),
+            _lib.stream_of(value))
     _lib.check(rc, "dfa3d_wms_deform_attn_backward")
 
 
@@ -238,7 +240,7 @@ def ms_deform_attn_forward(value, value_spatial_shapes, value_level_start_index,
         rc = _lib.lib().dfa3d_wms_deform_attn_forward(
             _lib.ptr(value), _lib.ptr(value_spatial_shapes), sw, _lib.ptr(value_level_start_index),
             _lib.ptr(sampling_locations), lw, _lib.ptr(attention_weights), None, _lib.ptr(out),
-            B, S, M, C, L, Q, P, _lib.dtype_code(value), _lib.stream_of(value))
+            B, S, M, C, L, Q, P, _lib.dtype_code(value), _lib.options(), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_wms_deform_attn_forward")
     return out
 
@@ -266,14 +268,14 @@ def ms_deform_attn_backward(value, value_spatial_shapes, value_level_start_index
     if grad_output.numel() == 0:
         return
     code = _lib.dtype_code(value)
-    ws_bytes = _lib.lib().dfa3d_wms_deform_attn_backward_workspace_bytes(B, S, M, C, L, Q, P, code)
+    ws_bytes = _lib.lib().dfa3d_wms_deform_attn_backward_workspace_bytes(B, S, M, C, L, Q, P, code, _lib.options())
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
     with torch.cuda.device(dev):
         rc = _lib.lib().dfa3d_wms_deform_attn_backward(
             _lib.ptr(value), _lib.ptr(value_spatial_shapes), sw, _lib.ptr(value_level_start_index),
             _lib.ptr(sampling_locations), lw, _lib.ptr(attention_weights), None, _lib.ptr(grad_output),
             _lib.ptr(grad_value), _lib.ptr(grad_sampling_loc), lw, _lib.ptr(grad_attn_weight), None,
-            _lib.ptr(workspace), ws_bytes, B, S, M, C, L, Q, P, code, _lib.stream_of(value))
+            _lib.ptr(workspace), ws_bytes, B, S, M, C, L, Q, P, code, _lib.options(), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_wms_deform_attn_backward")
 
 
@@ -317,7 +319,7 @@ def dfa3d_fused_forward(value, value_dpt_dist, value_spatial_shapes, value_level
             _lib.ptr(value), _lib.ptr(value_dpt_dist), _lib.ptr(value_spatial_shapes),
             _lib.ptr(value_level_start_index), _lib.ptr(sampling_locations), _lib.ptr(attention_weights),
             _lib.ptr(out), _lib.ptr(score), _lib.ptr(wu), B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2],
-            _lib.dtype_code(value), _lib.stream_of(value))
+            _lib.dtype_code(value), _lib.options(), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_fused_forward")
     return (out, score, wu) if need_weight_update else (out, score)
 
@@ -360,7 +362,8 @@ def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_leve
         return
     code = _lib.dtype_code(value)
     # scratch for the binned (LDS-accumulating) kernels; 0 bytes means the direct kernel is used
-    ws_bytes = _lib.lib().dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2], code)
+    ws_bytes = _lib.lib().dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2], code,
+                                                                _lib.options())
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
     with torch.cuda.device(dev):
         rc = _lib.lib().dfa3d_fused_backward(
@@ -369,5 +372,5 @@ def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_leve
             _lib.ptr(grad_output), _lib.ptr(grad_depth_score), _lib.ptr(grad_weight_update), _lib.ptr(grad_value),
             _lib.ptr(grad_value_dpt_dist), _lib.ptr(grad_sampling_loc), _lib.ptr(grad_attn_weight),
             _lib.ptr(workspace), ws_bytes, B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2], code,
-            _lib.stream_of(value))
+            _lib.options(), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_fused_backward")

@@ -3,8 +3,10 @@
 The library is the product: there is no CPU or pure-PyTorch fallback.  If the
 shared object is missing or a tensor is not on a GPU, the call raises.
 """
+import contextlib
 import ctypes
 import os
+import threading
 
 import torch
 
@@ -12,25 +14,32 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdfa3d_hip.so")
 
 DFA3D_F32, DFA3D_F64, DFA3D_BF16 = 0, 1, 2
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _P, _I = ctypes.c_void_p, ctypes.c_int
 _DIMS7 = [_I] * 7      # B S M (C|D) L Q P
 _DIMS8 = [_I] * 8      # B S M C D L Q P
 
+
+class LaunchOptions(ctypes.Structure):
+    """dfa3d_launch_options of include/dfa3d.h: how one call is laid out on the machine (never what it computes)."""
+    _fields_ = [("iters", _I), ("vec", _I), ("direct", _I), ("tile", _I), ("block", _I), ("pass_", _I), ("chunk", _I),
+                ("reserved", _I), ("event_binned", _P)]
+
+
+_O = ctypes.POINTER(LaunchOptions)
+
 # name -> argument types; every entry point returns int
 SIGNATURES = {
-    "dfa3d_ms_depth_score_sample_forward": [_P] * 5 + _DIMS7 + [_I, _P],
-    "dfa3d_ms_depth_score_sample_backward": [_P] * 8 + [ctypes.c_size_t] + _DIMS7 + [_I, _P],
-    "dfa3d_wms_deform_attn_forward": [_P, _P, _I, _P, _P, _I, _P, _P, _P] + _DIMS7 + [_I, _P],
+    "dfa3d_ms_depth_score_sample_forward": [_P] * 5 + _DIMS7 + [_I, _O, _P],
+    "dfa3d_ms_depth_score_sample_backward": [_P] * 8 + [ctypes.c_size_t] + _DIMS7 + [_I, _O, _P],
+    "dfa3d_wms_deform_attn_forward": [_P, _P, _I, _P, _P, _I, _P, _P, _P] + _DIMS7 + [_I, _O, _P],
     "dfa3d_wms_deform_attn_backward": [_P, _P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _P, ctypes.c_size_t]
-    + _DIMS7 + [_I, _P],
-    "dfa3d_fused_forward": [_P] * 9 + _DIMS8 + [_I, _I, _P],
-    "dfa3d_fused_backward": [_P] * 14 + [ctypes.c_size_t] + _DIMS8 + [_I, _I, _P],
+    + _DIMS7 + [_I, _O, _P],
+    "dfa3d_fused_forward": [_P] * 9 + _DIMS8 + [_I, _I, _O, _P],
+    "dfa3d_fused_backward": [_P] * 14 + [ctypes.c_size_t] + _DIMS8 + [_I, _I, _O, _P],
     "dfa3d_rebatch_gather": [_P, ctypes.c_longlong, ctypes.c_longlong, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "dfa3d_rebatch_combine": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
-    "dfa3d_set_tunable": [ctypes.c_char_p, _I],
-    "dfa3d_stream_copy": [_P, _P, ctypes.c_size_t, _P],
     "dfa3d_abi_version": [],
 }
 
@@ -54,7 +63,7 @@ def lib():
                            ("dfa3d_wms_deform_attn_backward_workspace_bytes", _DIMS7),
                            ("dfa3d_ms_depth_score_sample_backward_workspace_bytes", _DIMS7)):
             fn = getattr(handle, name)
-            fn.argtypes = dims + [_I]
+            fn.argtypes = dims + [_I, _O]
             fn.restype = ctypes.c_size_t
         handle.dfa3d_last_error.argtypes = []
         handle.dfa3d_last_error.restype = ctypes.c_char_p
@@ -70,8 +79,38 @@ def check(rc, name):
         raise RuntimeError(f"{name} failed with code {rc}: {msg}")
 
 
-def set_tunable(name, value):
-    check(lib().dfa3d_set_tunable(name.encode(), int(value)), "dfa3d_set_tunable")
+_tls = threading.local()
+
+
+@contextlib.contextmanager
+def launch_options(**fields):
+    """Every library call this thread makes inside the block carries these launch options
+    (``iters``, ``vec``, ``direct``, ``tile``, ``block``, ``pass_``, ``chunk``, ``event_binned``); nested blocks
+    add to the enclosing ones.  Outside any block calls pass NULL: the defaults."""
+    merged = dict(getattr(_tls, "fields", {}))
+    for k, v in fields.items():
+        if k == "pass":
+            k = "pass_"
+        if k not in dict(LaunchOptions._fields_) or k == "reserved":
+            raise TypeError(f"unknown launch option {k!r}")
+        merged[k] = v
+    saved = getattr(_tls, "fields", None)
+    _tls.fields = merged
+    try:
+        yield
+    finally:
+        if saved is None:
+            del _tls.fields
+        else:
+            _tls.fields = saved
+
+
+def options():
+    """ctypes argument for the ``opts`` parameter of an entry point: NULL, or the calling thread's current options."""
+    fields = getattr(_tls, "fields", None)
+    if not fields:
+        return None
+    return ctypes.pointer(LaunchOptions(**fields))
 
 
 def dtype_code(t):

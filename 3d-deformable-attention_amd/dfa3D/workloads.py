@@ -31,6 +31,7 @@ class Workload:
     loc_std: float = 0.15
     depth: str = "softmax"      # "softmax" of N(0, sigma) logits or "peaky" (8*onehot + N(0,1))
     depth_sigma: float = 1.0
+    attn: str = "softmax"       # "softmax" over levels x points, or "rand": U[0,1) weights that do not sum to 1
 
     @property
     def L(self):
@@ -78,12 +79,15 @@ WORKLOADS = {
     "base": Workload("base", B=6, Q=10000, levels=_BASE_LEVELS, D=64, P=8, depth_sigma=2.0),
     # base shape, GT-depth-like peaky distributions (used with bf16 storage)
     "base_peaky": Workload("base_peaky", B=6, Q=10000, levels=_BASE_LEVELS, D=64, P=8, depth="peaky"),
+    # the operands of the reference's own test (unittest_DFA3D.py:43-56): 112 depth bins, 9502 queries, attention
+    # weights drawn from U[0,1) without normalisation
+    "unittest": Workload("unittest", B=6, Q=9502, levels=_BASE_LEVELS, D=112, P=8, attn="rand"),
     # dense BEV grid, clustered locations
     "dense": Workload("dense", B=6, Q=40000, levels=_BASE_LEVELS, D=128, P=8, loc="normal",
                       loc_lo=-0.1, loc_hi=1.1, depth_sigma=2.0),
 }
 
-SEEDS = {"unit": 1, "small": 2, "base": 3, "base_peaky": 4, "dense": 5}
+SEEDS = {"unit": 1, "small": 2, "base": 3, "base_peaky": 4, "dense": 5, "unittest": 6}
 
 
 def scaled(w: Workload, B=None, Q=None, name=None) -> Workload:
@@ -112,7 +116,10 @@ def make_inputs(w: Workload, seed=None, dtype=torch.float32, device="cpu", grad_
         loc.clamp_(w.loc_lo, w.loc_hi)
     else:
         loc = torch.rand(B, Q, M, L, P, 3, generator=g, dtype=torch.float32) * (w.loc_hi - w.loc_lo) + w.loc_lo
-    attn = torch.randn(B, Q, M, L * P, generator=g, dtype=torch.float32).softmax(-1).view(B, Q, M, L, P)
+    if w.attn == "rand":
+        attn = torch.rand(B, Q, M, L, P, generator=g, dtype=torch.float32)
+    else:
+        attn = torch.randn(B, Q, M, L * P, generator=g, dtype=torch.float32).softmax(-1).view(B, Q, M, L, P)
     out = {
         "value": value, "value_dpt_dist": dist,
         "spatial_shapes": torch.tensor([[h, w_, D] for h, w_ in w.levels], dtype=torch.int64),

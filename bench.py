@@ -1,7 +1,9 @@
 #!/usr/bin/env python3
 """Benchmark of the DFA3D operator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload base|small|unit|dense|base_bf16]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload base|small|unit|dense|base_bf16|unittest]
+    python bench.py --micro                      yardsticks of the machine (copy, bare gathers, LDS atomics, XCD map)
+    python bench.py --summarize NAME DIR [DIR..] tables from rocprofv3 output directories -> profiles/NAME.txt
 
 A step is one forward + backward of the one-stage autograd Function
 (MultiScale3DDeformableAttnFunction.apply -> torch.autograd.grad) over one batch of synthetic
@@ -10,38 +12,42 @@ BEVFormer-shaped operands already resident in HBM.  Prints ONE JSON line:
   metric/value   sampled points (B*Q*M*L*P) per second of forward+backward, whole job
   ms_per_step    forward+backward through autograd (includes its allocations and zero fills)
   kernels        launch durations measured with events on the launch stream: the forward kernel, the
-                 backward's binning kernels (as a group) and its tile kernel, with the algorithmic
-                 GB/s (each operand read once, each result written once) they amount to
-  roofline       the same for the dominant (longest) kernel, against MI355X's 8 TB/s HBM peak
+                 backward's binning kernels (as a group) and its tile kernel (the library records an event
+                 between the two groups of the SAME call), with the algorithmic GB/s (each operand read once,
+                 each result written once) they amount to
+  roofline       the same for the dominant (longest) kernel, against MI355X's 8 TB/s HBM peak; `traffic` is
+                 the HBM-side byte count of that kernel from profiles/hbm_traffic.json when that file was
+                 written for the kernel sources as they are now, else null
+  roofline_whole_backward   all launches of one backward call against the backward's algorithmic bytes
+  attainable_gbs what a plain streaming copy of 1 GiB reaches on this GPU (read + write bytes per second)
   cpu_baseline   the scalar C restatement of the operator (oracle/) on the host cores, on a
                  bounded sample of the same workload
 """
 import argparse
+import ctypes
+import glob
+import hashlib
 import json
 import os
+import re
 import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.join(ROOT, "3d-deformable-attention_amd"))
+PKG = os.path.join(ROOT, "3d-deformable-attention_amd")
+sys.path.insert(0, PKG)
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
-
-# HBM-side bytes per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each
-# scaled by what the same counter reads for the library's plain 1 GiB streaming copy (profiles/).
-MEASURED_TRAFFIC_BYTES = {
-    # profiles/fwd_attention_and_tile_backward_base_fp32.txt
-    ("base", "forward"): 5.22e9,
-    ("base", "backward_tile"): 4.15e9,
-}
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+OPTION_NAMES = ("iters", "vec", "direct", "tile", "block", "pass", "chunk")
 
 
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="base")
     ap.add_argument("--kernel-reps", type=int, default=20, help="launches per kernel for the event timings")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
@@ -49,10 +55,235 @@ def parse():
                     help="also run one plain streaming copy of this many MiB (yardstick for profiler HBM counters)")
     ap.add_argument("--no-variants", dest="variants", action="store_false",
                     help="skip the timings of the two-stage, shared-distribution and plain-attention entry points")
-    ap.add_argument("--tunable", action="append", default=[], metavar="NAME=VALUE", help="library launch tunable")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="launch option for every library call (%s)" % ", ".join(OPTION_NAMES))
+    ap.add_argument("--micro", action="store_true", help="run the yardstick kernels instead of the operator")
+    ap.add_argument("--summarize", nargs="+", metavar=("NAME", "DIR"),
+                    help="write profiles/NAME.txt (and profiles/hbm_traffic.json) from rocprofv3 output directories")
+    ap.add_argument("--summarize-command", action="append", default=[],
+                    help="with --summarize: a command line to quote in the summary's header (repeatable)")
     return ap.parse_args()
 
 
+def sources_digest():
+    """SHA-256 over the kernel sources: what a traffic figure from the profiler is valid for."""
+    h = hashlib.sha256()
+    for path in sorted(glob.glob(os.path.join(PKG, "csrc", "*.hip")) + glob.glob(os.path.join(PKG, "csrc", "*.h"))):
+        h.update(os.path.basename(path).encode())
+        h.update(open(path, "rb").read())
+    return h.hexdigest()
+
+
+def recorded_traffic(workload):
+    """{kernel key: HBM-side bytes per launch} from profiles/hbm_traffic.json, or {} when the file is missing,
+    holds nothing for this workload or was written for other kernel sources."""
+    try:
+        doc = json.load(open(TRAFFIC_JSON))
+    except (OSError, ValueError):
+        return {}, "no profiles/hbm_traffic.json"
+    rec = doc.get(workload)
+    if not rec:
+        return {}, f"profiles/hbm_traffic.json holds nothing for workload {workload}"
+    if rec.get("sources_sha256") != sources_digest():
+        return {}, "profiles/hbm_traffic.json was written for other kernel sources (stale)"
+    return {k: v["fetch_bytes"] + v["write_bytes"] for k, v in rec["kernels"].items()}, rec.get("summary", "")
+
+
+# ------------------------------------------------------------------------------------------------
+# measure library (yardstick kernels)
+# ------------------------------------------------------------------------------------------------
+def measure_lib():
+    path = os.path.join(PKG, "dfa3D", "libdfa3d_measure.so")
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: build it with `python 3d-deformable-attention_amd/build.py`")
+    h = ctypes.CDLL(path)
+    P, I, Z = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    h.dfa3d_measure_stream_copy.argtypes = [P, P, Z, P]
+    h.dfa3d_measure_xcd_map.argtypes = [P, I, I, I, P]
+    h.dfa3d_measure_row_gather.argtypes = [P, Z, I, I, I, I, P, P]
+    h.dfa3d_measure_pair_gather.argtypes = [P, Z, I, I, I, P, P]
+    h.dfa3d_measure_lds_atomics.argtypes = [I, I, I, P, P]
+    return h
+
+
+def copy_bandwidth(torch, mib=1024, reps=5):
+    """GB/s (bytes read + bytes written) of a plain streaming copy: the attainable ceiling on this GPU."""
+    m = measure_lib()
+    dev = torch.device("cuda:0")
+    n = mib << 20
+    src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+    def run():
+        rc = m.dfa3d_measure_stream_copy(dst.data_ptr(), src.data_ptr(), n, stream)
+        assert rc == 0, rc
+
+    run()
+    ms, best = event_time(run, reps)
+    return 2 * n / (best * 1e-3) / 1e9
+
+
+def micro():
+    """Yardsticks: what the machine does for the bare access patterns of the kernels."""
+    import torch
+    m = measure_lib()
+    dev = torch.device("cuda:0")
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    sink = torch.zeros(64, dtype=torch.uint8, device=dev)
+    props = torch.cuda.get_device_properties(0)
+    cus = props.multi_processor_count
+    out = {"device": props.name, "compute_units": cus, "copy_gbs": round(copy_bandwidth(torch), 1)}
+
+    # which XCD do the workgroups of a launch land on?  (the kernels tie heads to XCDs through block id % 8)
+    maps = {}
+    for blocks, threads in ((4096, 256), (512, 512), (60000, 256)):
+        buf = torch.full((blocks,), -1, dtype=torch.int32, device=dev)
+        rows = []
+        for _ in range(3):
+            rc = m.dfa3d_measure_xcd_map(buf.data_ptr(), blocks, threads, 20000, stream)
+            assert rc == 0, rc
+            torch.cuda.synchronize()
+            x = buf.cpu()
+            blk = torch.arange(blocks) % 8
+            hist = torch.zeros(8, 8, dtype=torch.int64)
+            hist.index_put_((blk, x.long().clamp(0, 7)), torch.ones(blocks, dtype=torch.int64), accumulate=True)
+            rows.append({"on_diagonal": int(hist.diag().sum()), "blocks": blocks,
+                         "xcd_of_block_mod_8": hist.argmax(1).tolist(), "xcds_seen": int(x.unique().numel())})
+        maps[f"{blocks}x{threads}"] = rows
+    out["xcd_map"] = maps
+
+    # random whole-row gathers (the value-row gathers of the forward) against the footprint they are drawn from
+    src = torch.zeros(1 << 30, dtype=torch.uint8, device=dev)
+    blocks, iters = cus * 32, 64
+    rows_tbl = []
+    for row_bytes in (128, 256, 64):
+        lanes = row_bytes // 16
+        for mb in (2, 16, 64, 256, 1024):
+            rows = (mb << 20) // row_bytes
+            for infl in ((8,) if row_bytes != 128 else (1, 4, 8)):
+                fn = lambda: m.dfa3d_measure_row_gather(src.data_ptr(), rows, row_bytes, infl, blocks, iters,
+                                                        sink.data_ptr(), stream)
+                assert fn() == 0
+                _, best = event_time(fn, 3)
+                n_rows = blocks * 256 // lanes * iters * infl
+                rows_tbl.append({"row_bytes": row_bytes, "footprint_mib": mb, "in_flight": infl,
+                                 "tb_per_s": round(n_rows * row_bytes / (best * 1e-3) / 1e12, 2),
+                                 "ps_per_row": round(best * 1e-3 / n_rows * 1e12, 1),
+                                 "clocks_per_row_per_cu": round(best * 1e-3 / n_rows * cus * 2.4e9, 2)})
+    out["row_gather"] = rows_tbl
+    # random 8-byte gathers, 64 different lines per wavefront instruction (the depth taps)
+    pair_tbl = []
+    for mb in (2, 16, 64, 256, 1024):
+        for infl in (1, 4, 8):
+            fn = lambda: m.dfa3d_measure_pair_gather(src.data_ptr(), mb << 20, infl, blocks, iters, sink.data_ptr(), stream)
+            assert fn() == 0
+            _, best = event_time(fn, 3)
+            n = blocks * 256 * iters * infl
+            pair_tbl.append({"footprint_mib": mb, "in_flight": infl, "g_loads_per_s": round(n / (best * 1e-3) / 1e9, 1),
+                             "ps_per_load": round(best * 1e-3 / n * 1e12, 1),
+                             "clocks_per_load_per_cu": round(best * 1e-3 / n * cus * 2.4e9, 2)})
+    out["pair_gather"] = pair_tbl
+    del src
+    names = ["float add, one bank per lane", "float add, random", "float add, one address",
+             "int add returning, random", "int add, random", "int exchange, random"]
+    lds = []
+    for mode, name in enumerate(names):
+        blocks_l, iters_l = 2048, 2000
+        fn = lambda: m.dfa3d_measure_lds_atomics(mode, blocks_l, iters_l, sink.data_ptr(), stream)
+        assert fn() == 0
+        _, best = event_time(fn, 3)
+        n = blocks_l * 256 * iters_l
+        lds.append({"pattern": name, "lanes_per_clock_per_cu": round(n / (best * 1e-3) / 2.4e9 / cus, 3)})
+    out["lds_atomics"] = lds
+    print(json.dumps(out))
+
+
+# ------------------------------------------------------------------------------------------------
+# rocprofv3 summaries
+# ------------------------------------------------------------------------------------------------
+KERNEL_KEYS = (("fwd_attention_kernel", "forward"), ("tile_backward_kernel", "backward_tile"),
+               ("bin_points_kernel<1>", "bin_fill"), ("bin_points_kernel<0>", "bin_count"))
+
+
+def short_name(n):
+    n = re.sub(r"\(.*", "", n)
+    return n.replace("dfa3d::", "").replace("void ", "").replace("(anonymous namespace)::", "")[:92]
+
+
+def summarize(name, dirs, commands):
+    """Per-kernel tables from rocprofv3's rocpd databases (kernel durations; counters per dispatch) as text under
+    profiles/, and the HBM-side bytes of the operator's kernels (FETCH_SIZE / WRITE_SIZE, each scaled by what the
+    same counter reads for the yardstick copy of known size in the same run) into profiles/hbm_traffic.json."""
+    import sqlite3
+    lines = [f"# {c}" for c in commands]
+    scale, raw, workload = {}, {}, None
+    for d in dirs:
+        for db in sorted(glob.glob(os.path.join(d, "**", "*.db"), recursive=True)):
+            c = sqlite3.connect(db)
+            rows = c.execute("select name, count(*), avg(end-start), min(end-start), max(end-start), sum(end-start) "
+                             "from kernels group by name order by 6 desc").fetchall()
+            tot = sum(r[5] for r in rows) or 1
+            lines += ["", f"## {os.path.relpath(db, ROOT)}: kernel durations",
+                      f"{'kernel':94s} {'calls':>5s} {'avg_us':>10s} {'min_us':>10s} {'max_us':>10s} {'pct':>6s}"]
+            for n, k, a, mi, ma, s in rows[:16]:
+                lines.append(f"{short_name(n):94s} {k:5d} {a / 1e3:10.1f} {mi / 1e3:10.1f} {ma / 1e3:10.1f} {100 * s / tot:6.1f}")
+            try:
+                rows = c.execute("select kernel_name, counter_name, count(*), avg(value), min(value), max(value) from "
+                                 "counters_collection group by kernel_name, counter_name order by 1, 2").fetchall()
+            except sqlite3.Error:
+                rows = []
+            if rows:
+                lines += ["", f"## {os.path.relpath(db, ROOT)}: counters per dispatch (raw)",
+                          f"{'kernel':94s} {'counter':>22s} {'n':>4s} {'avg':>16s} {'min':>16s} {'max':>16s}"]
+            for n, cn, k, a, mi, ma in rows:
+                if "dfa3d" not in n and "stream_copy" not in n:
+                    continue
+                lines.append(f"{short_name(n):94s} {cn:>22s} {k:4d} {a:16.1f} {mi:16.1f} {ma:16.1f}")
+                if "stream_copy_kernel" in n and cn in ("FETCH_SIZE", "WRITE_SIZE"):
+                    scale[cn] = a
+                for frag, key in KERNEL_KEYS:
+                    if frag in n and cn in ("FETCH_SIZE", "WRITE_SIZE"):
+                        raw.setdefault(key, {})[cn] = a
+            c.close()
+    mib = None
+    for cmd in commands:
+        m = re.search(r"--workload\s+(\S+)", cmd)
+        if m:
+            workload = m.group(1)
+        m = re.search(r"--calibration-copy-mib\s+(\d+)", cmd)
+        if m:
+            mib = int(m.group(1))
+    workload = workload or "base"
+    copy_kib = (mib << 10) if mib else None
+    traffic = {}
+    if copy_kib and "FETCH_SIZE" in scale and "WRITE_SIZE" in scale:
+        f_scale, w_scale = copy_kib / scale["FETCH_SIZE"], copy_kib / scale["WRITE_SIZE"]
+        lines += ["", f"## HBM-side bytes per launch: counter (KiB) x 1024 x scale factor; the yardstick copy moves "
+                      f"{copy_kib} KiB each way, FETCH_SIZE reads {scale['FETCH_SIZE']:.0f} for it (factor {f_scale:.3f}), "
+                      f"WRITE_SIZE {scale['WRITE_SIZE']:.0f} (factor {w_scale:.3f})"]
+        for key, v in raw.items():
+            if "FETCH_SIZE" in v and "WRITE_SIZE" in v:
+                fb, wb = v["FETCH_SIZE"] * 1024 * f_scale, v["WRITE_SIZE"] * 1024 * w_scale
+                traffic[key] = {"fetch_bytes": round(fb), "write_bytes": round(wb)}
+                lines.append(f"{key:16s} fetch {fb / 1e9:7.3f} GB   write {wb / 1e9:7.3f} GB   total {(fb + wb) / 1e9:7.3f} GB")
+    out_txt = os.path.join(ROOT, "profiles", name + ".txt")
+    with open(out_txt, "w") as f:
+        f.write("\n".join(lines) + "\n")
+    print("wrote", out_txt)
+    if traffic:
+        try:
+            doc = json.load(open(TRAFFIC_JSON))
+        except (OSError, ValueError):
+            doc = {}
+        doc[workload] = {"sources_sha256": sources_digest(), "summary": f"profiles/{name}.txt", "kernels": traffic}
+        with open(TRAFFIC_JSON, "w") as f:
+            json.dump(doc, f, indent=1, sort_keys=True)
+            f.write("\n")
+        print("updated", TRAFFIC_JSON)
+
+
+# ------------------------------------------------------------------------------------------------
 def variant_timings(_ext, torch, value, dist, shapes, lsi, loc, attn, go, reps):
     """Event timings (ms, average) of the other entry points on the same operands: the reference's two-stage
     composition, the caller-shaped call (one distribution for all heads, weight_update instead of the score
@@ -167,6 +398,9 @@ def cpu_baseline(w, budget_s):
 
 def main():
     a = parse()
+    if a.summarize:
+        summarize(a.summarize[0], a.summarize[1:], a.summarize_command)
+        return
     if a.gpus != 1:
         print(f"bench.py: this build runs on ONE GPU (one MI355X per box); --gpus {a.gpus} is not supported. "
               "The operator shards over the batch (camera) dimension without any exchange.", file=sys.stderr)
@@ -179,11 +413,22 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP kernels are the product and there is no fallback", file=sys.stderr)
         sys.exit(3)
+    if a.micro:
+        micro()
+        return
     L_ = _lib.lib()
-    for t in a.tunable:
+    user_options = {}
+    for t in a.option:
         name, val = t.split("=")
-        _lib.set_tunable(name, int(val))
+        if name not in OPTION_NAMES:
+            print(f"bench.py: unknown launch option {name}", file=sys.stderr)
+            sys.exit(2)
+        user_options[name] = int(val)
+    with _lib.launch_options(**user_options):
+        run(a, torch, _ext, _lib, L_, MultiScale3DDeformableAttnFunction, WORKLOADS, make_inputs, user_options)
 
+
+def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
     bf16 = a.workload.endswith("_bf16")
     wname = "base_peaky" if a.workload == "base_bf16" else a.workload
     w = WORKLOADS[wname]
@@ -198,24 +443,19 @@ def main():
     e_v = 2 if bf16 else 4
     fwd_bytes, bwd_bytes = w.forward_bytes(e_v, e_v), w.backward_bytes(e_v, e_v)
 
-    if a.calibration_copy_mib > 0:
-        n = a.calibration_copy_mib << 20
-        src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
-        dst = torch.empty_like(src)
-        for _ in range(2):
-            _lib.check(L_.dfa3d_stream_copy(_lib.ptr(dst), _lib.ptr(src), n, _lib.stream_of(src)), "dfa3d_stream_copy")
-        torch.cuda.synchronize()
-        del src, dst
+    attainable = copy_bandwidth(torch, mib=max(a.calibration_copy_mib, 1024), reps=5)
+    if a.calibration_copy_mib > 0:       # one more copy of exactly the stated size, for the profiler
+        copy_bandwidth(torch, mib=a.calibration_copy_mib, reps=1)
 
     leaves = [t.requires_grad_() for t in (value, dist, loc, attn)]
 
     def step():
-        out, _ = MultiScale3DDeformableAttnFunction.apply(leaves[0], leaves[1], shapes, lsi, leaves[2], leaves[3], 64)
+        out, _ = F1.apply(leaves[0], leaves[1], shapes, lsi, leaves[2], leaves[3], 64)
         return torch.autograd.grad(out, leaves, go)
 
     def fwd_only():
         with torch.no_grad():
-            return MultiScale3DDeformableAttnFunction.apply(value, dist, shapes, lsi, loc, attn, 64)
+            return F1.apply(value, dist, shapes, lsi, loc, attn, 64)
 
     for _ in range(a.warmup):
         step()
@@ -251,20 +491,28 @@ def main():
     D = dist.shape[3]
     _, Q, _, L, P, _ = loc.shape
     code = _lib.dtype_code(value)
-    gv = torch.zeros(value.shape, dtype=torch.float32, device=dev)
-    gd = torch.zeros(dist.shape, dtype=torch.float32, device=dev)
+    gdt = torch.float32
+    gv = torch.zeros(value.shape, dtype=gdt, device=dev)
+    gd = torch.zeros(dist.shape, dtype=gdt, device=dev)
     gl = torch.empty_like(loc)
     ga = torch.empty_like(attn)
     vd, dd, ld, ad = value.detach(), dist.detach(), loc.detach(), attn.detach()
-    ws_bytes = L_.dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, dist.shape[2], code)
+    ws_bytes = L_.dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, dist.shape[2], code, _lib.options())
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     stream = _lib.stream_of(value)
+    # the library records this event between the binning kernels and the tile kernel of a binned backward
+    mid = torch.cuda.Event(enable_timing=True)
+    mid.record()
+    torch.cuda.synchronize()
+    mid_handle = mid.cuda_event
+    assert mid_handle, "torch did not create the event"
 
-    def backward_call():
+    def backward_call(opts=None):
         _lib.check(L_.dfa3d_fused_backward(
             _lib.ptr(vd), _lib.ptr(dd), _lib.ptr(shapes), _lib.ptr(lsi), _lib.ptr(ld), _lib.ptr(ad), _lib.ptr(go), None,
             None, _lib.ptr(gv), _lib.ptr(gd), _lib.ptr(gl), _lib.ptr(ga), _lib.ptr(ws) if ws_bytes else None, ws_bytes,
-            B, S, M, C, D, L, Q, P, dist.shape[2], code, stream), "dfa3d_fused_backward")
+            B, S, M, C, D, L, Q, P, dist.shape[2], code, opts if opts is not None else _lib.options(), stream),
+            "dfa3d_fused_backward")
 
     def zero():
         gv.zero_()
@@ -273,45 +521,55 @@ def main():
     fwd_ms, fwd_best = event_time(lambda: _ext.dfa3d_fused_forward(vd, dd, shapes, lsi, ld, ad, 64), a.kernel_reps)
     bwd_all_ms, bwd_all_best = event_time(backward_call, a.kernel_reps, prep=zero)
     fill_ms, _ = event_time(zero, a.kernel_reps)
+    traffic, traffic_note = ({}, "launch options given: recorded traffic does not apply") if user_options \
+        else recorded_traffic(a.workload)
 
     def entry(name, ms, best, nbytes, key=None):
         gbs = nbytes / (ms * 1e-3) / 1e9
         e = {"kernel": name, "avg_ms": round(ms, 4), "min_ms": round(best, 4), "algorithmic_bytes": nbytes,
              "achieved_gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
              "points_per_s": w.points / (ms * 1e-3)}
-        traffic = MEASURED_TRAFFIC_BYTES.get((a.workload, key)) if not bf16 else None
-        if traffic:
-            # bytes the hardware counters saw on the memory side of the L2, over the time measured here
-            e["counter_traffic_gbs"] = round(traffic / (ms * 1e-3) / 1e9, 1)
-            e["counter_traffic_frac_of_hbm_peak"] = round(traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        if traffic.get(key):
+            # bytes the hardware counters saw on the memory side of the L2: above the algorithmic bytes = lines
+            # fetched or written more than once
+            e["hbm_side_bytes"] = traffic[key]
+            e["hbm_side_bytes_over_algorithmic"] = round(traffic[key] / nbytes, 2)
         return e
 
     kernels = {"forward": entry("fwd_attention_kernel (depth score + attention, one launch)", fwd_ms, fwd_best, fwd_bytes,
                                 "forward")}
+    whole_bwd = {"bound": "hbm", "launches": "every kernel of one dfa3d_fused_backward call", "avg_ms": round(bwd_all_ms, 4),
+                 "achieved": round(bwd_bytes / (bwd_all_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                 "frac": round(bwd_bytes / (bwd_all_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     if ws_bytes:
-        # binning kernels alone, then the tile kernel alone on the workspace they prepared
-        _lib.set_tunable("bwd_stage", 1)
-        bin_ms, bin_best = event_time(backward_call, a.kernel_reps)
-
-        def prepare_tile():
+        # the two parts of the SAME backward call: [start .. event recorded by the library] = binning kernels,
+        # [that event .. end] = tile kernel (plus the head sum for a shared distribution)
+        fields = dict(user_options)
+        if "pass" in fields:
+            fields["pass_"] = fields.pop("pass")
+        opts = ctypes.pointer(_lib.LaunchOptions(event_binned=mid_handle, **fields))
+        bin_t, tile_t = [], []
+        for _ in range(a.kernel_reps):
             zero()
-            _lib.set_tunable("bwd_stage", 1)
-            backward_call()
-            _lib.set_tunable("bwd_stage", 2)
-
-        tile_ms, tile_best = event_time(backward_call, a.kernel_reps, prep=prepare_tile)
-        _lib.set_tunable("bwd_stage", 0)
-        kernels["backward_tile"] = entry("tile_backward_kernel (all gradients, one launch)", tile_ms, tile_best, bwd_bytes,
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            backward_call(opts)
+            e1.record()
+            e1.synchronize()
+            bin_t.append(e0.elapsed_time(mid))
+            tile_t.append(mid.elapsed_time(e1))
+        bin_ms, tile_ms = sum(bin_t) / len(bin_t), sum(tile_t) / len(tile_t)
+        kernels["backward_tile"] = entry("tile_backward_kernel (all gradients, one launch)", tile_ms, min(tile_t), bwd_bytes,
                                          "backward_tile")
         kernels["backward_binning"] = {"kernel": "plan_and_clear + bin_points<0> + bin_scan + bin_points<1> (4 launches)",
-                                       "avg_ms": round(bin_ms, 4), "min_ms": round(bin_best, 4)}
+                                       "avg_ms": round(bin_ms, 4), "min_ms": round(min(bin_t), 4)}
         dom = "backward_tile" if tile_ms >= fwd_ms else "forward"
     else:
         kernels["backward_direct"] = entry("bwd_attention_kernel (device-memory atomics)", bwd_all_ms, bwd_all_best, bwd_bytes)
         dom = "backward_direct" if bwd_all_ms >= fwd_ms else "forward"
     k = kernels[dom]
     roofline = {"bound": "hbm", "kernel": k["kernel"], "achieved": k["achieved_gbs"], "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": k["frac_of_hbm_peak"], "traffic": MEASURED_TRAFFIC_BYTES.get((a.workload, dom))}
+                "unit": "GB/s", "frac": k["frac_of_hbm_peak"], "traffic": traffic.get(dom), "traffic_source": traffic_note}
 
     result = {
         "metric": "dfa3d_fwd_bwd_sampled_points_per_s",
@@ -323,14 +581,17 @@ def main():
         "dtype": "bf16" if bf16 else "f32", "data": "synthetic",
         "config": {"workload": f"{a.workload}: B={w.B} Q={w.Q} M={w.M} C={w.C} L={w.L} "
                                f"levels={'/'.join(f'{h}x{x}' for h, x in w.levels)} D={w.D} P={w.P} "
-                               f"({w.points} sampled points), one-stage Function forward+backward"},
+                               f"({w.points} sampled points), one-stage Function forward+backward",
+                   "launch_options": user_options},
         "step_ms_spread": step_spread,
         "fwd_ms": round(fwd_api_ms, 4), "fwd_kernel_ms": round(fwd_ms, 4),
         "bwd_launches_ms": round(bwd_all_ms, 4), "grad_zero_fill_ms": round(fill_ms, 4),
         "fwd_points_per_s": w.points / (fwd_api_ms * 1e-3),
         "fwd_frac_of_hbm_peak": kernels["forward"]["frac_of_hbm_peak"],
+        "attainable_gbs": round(attainable, 1),
         "kernels": kernels,
         "roofline": roofline,
+        "roofline_whole_backward": whole_bwd,
     }
     if a.variants:
         result["variants"] = variant_timings(_ext, torch, vd, dd, shapes, lsi, ld, ad, go, max(a.kernel_reps // 2, 3))

@@ -3,8 +3,9 @@
  *
  * C ABI of the shared library.  Every pointer except `stream` is a DEVICE pointer
  * into memory the caller owns; the library allocates nothing, keeps no state
- * besides a thread-local error string and the launch tunables, launches on `stream` (a hipStream_t, NULL
- * = the default stream) and returns without synchronising.  Return value: 0 on
+ * besides a thread-local error string and per-device launch attributes it has looked up once,
+ * launches on `stream` (a hipStream_t, NULL = the default stream) and returns without
+ * synchronising.  Return value: 0 on
  * success, a negative DFA3D_E* code for a rejected argument, a positive
  * hipError_t for a failed launch; dfa3d_last_error() describes the last failure
  * of the calling thread.
@@ -44,6 +45,22 @@ extern "C" {
 
 #define DFA3D_MAX_LEVELS 16
 
+/* Launch options of ONE call.  NULL, or a zero-filled structure, means the defaults.  They choose how the
+ * work is laid out on the machine and never what is computed: results agree up to floating-point
+ * summation order of grad_value / grad_dist, whatever the values. */
+typedef struct dfa3d_launch_options {
+  int iters;    /* groups of units each wavefront walks through; 0 = 1, at most 64 */
+  int vec;      /* channels per lane in the row gathers: 0 = automatic, 1, 2 or 4 (8: tile kernels only) */
+  int direct;   /* non-zero: a backward ignores its workspace and adds straight into device memory */
+  int tile;     /* binned backward: tile edge in pixels as ty*100+tx, 0 = automatic */
+  int block;    /* binned backward: threads per tile workgroup, 256 or 0/512 */
+  int pass;     /* binned backward: points a tile workgroup takes per pass, 64, 128 or 256; 0 = automatic */
+  int chunk;    /* binned backward: points of one tile handled by one work item, 0 = 4096 */
+  int reserved; /* must be 0 */
+  void *event_binned;   /* a hipEvent_t, or NULL: a binned backward records it on `stream` between its binning
+                         * kernels and its tile kernel, so that a profiler can time the two parts of the call */
+} dfa3d_launch_options;
+
 #define DFA3D_EINVAL (-1)   /* null pointer, non-positive dimension, bad stride or dtype */
 #define DFA3D_ERANGE (-2)   /* a dimension exceeds what the kernels index (see dfa3d_last_error) */
 
@@ -54,7 +71,7 @@ extern "C" {
 int dfa3d_ms_depth_score_sample_forward(
     const void *dist, const int64_t *shapes3, const int64_t *level_start, const void *loc3,
     void *score,
-    int B, int S, int M, int D, int L, int Q, int P, int dtype, void *stream);
+    int B, int S, int M, int D, int L, int Q, int P, int dtype, const dfa3d_launch_options *opts, void *stream);
 
 /* Stage 1 backward.  `grad_dist` is ACCUMULATED into (caller zero-fills); every element of
  * `grad_loc3` is overwritten, its x and y components with 0.  `workspace` as for
@@ -67,9 +84,9 @@ int dfa3d_ms_depth_score_sample_backward(
     const void *grad_score,
     void *grad_dist, void *grad_loc3,
     void *workspace, size_t workspace_bytes,
-    int B, int S, int M, int D, int L, int Q, int P, int dtype, void *stream);
+    int B, int S, int M, int D, int L, int Q, int P, int dtype, const dfa3d_launch_options *opts, void *stream);
 size_t dfa3d_ms_depth_score_sample_backward_workspace_bytes(int B, int S, int M, int D, int L, int Q, int P,
-                                                            int dtype);
+                                                            int dtype, const dfa3d_launch_options *opts);
 
 /* Stage 2 forward: depth-weighted multi-scale deformable attention.  Writes every element of
  * `out`.  `score` == NULL stands for scores that are all 1: plain multi-scale deformable attention,
@@ -81,7 +98,7 @@ int dfa3d_wms_deform_attn_forward(
     const void *value, const int64_t *shapes, int shape_stride, const int64_t *level_start,
     const void *loc, int loc_stride, const void *attn, const void *score,
     void *out,
-    int B, int S, int M, int C, int L, int Q, int P, int dtype, void *stream);
+    int B, int S, int M, int C, int L, int Q, int P, int dtype, const dfa3d_launch_options *opts, void *stream);
 
 /* Stage 2 backward.  `grad_value` must be zero on entry and holds the gradient on return;
  * `grad_loc` (B,Q,M,L,P,grad_loc_stride) gets its first two components overwritten, `grad_attn` and
@@ -95,8 +112,9 @@ int dfa3d_wms_deform_attn_backward(
     const void *loc, int loc_stride, const void *attn, const void *score, const void *grad_out,
     void *grad_value, void *grad_loc, int grad_loc_stride, void *grad_attn, void *grad_score,
     void *workspace, size_t workspace_bytes,
-    int B, int S, int M, int C, int L, int Q, int P, int dtype, void *stream);
-size_t dfa3d_wms_deform_attn_backward_workspace_bytes(int B, int S, int M, int C, int L, int Q, int P, int dtype);
+    int B, int S, int M, int C, int L, int Q, int P, int dtype, const dfa3d_launch_options *opts, void *stream);
+size_t dfa3d_wms_deform_attn_backward_workspace_bytes(int B, int S, int M, int C, int L, int Q, int P, int dtype,
+                                                      const dfa3d_launch_options *opts);
 
 /* Both stages in one kernel: what the reference's one-stage autograd Function does with two
  * native calls and two slice copies
@@ -113,7 +131,8 @@ int dfa3d_fused_forward(
     const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
     const void *loc3, const void *attn,
     void *out, void *score, void *weight_update,
-    int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype, void *stream);
+    int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype,
+    const dfa3d_launch_options *opts, void *stream);
 
 /* Backward of dfa3d_fused_forward (…_function.py:306-352: two native calls, six zero fills and
  * a host synchronisation in the reference).  The depth scores are recomputed from `dist`, not
@@ -135,14 +154,15 @@ int dfa3d_fused_backward(
     const void *grad_weight_update,
     void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn,
     void *workspace, size_t workspace_bytes,
-    int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype, void *stream);
+    int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype,
+    const dfa3d_launch_options *opts, void *stream);
 
 /* Scratch bytes dfa3d_fused_backward wants for these dimensions; 0 when the binned path does not
  * apply (DFA3D_F64, rows too long for LDS tiles, more than 2^31 points, invalid dimensions).  With
  * dist_heads = 1 this includes B*S*M*D floats: grad_dist is formed per head and summed over the heads
  * by a last kernel. */
 size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads,
-                                            int dtype);
+                                            int dtype, const dfa3d_launch_options *opts);
 
 /* Camera re-batching around the operator, as DFA3D-BEVFormer's spatial cross-attention does it in python
  * loops over batch x cameras
@@ -165,24 +185,6 @@ int dfa3d_rebatch_combine(const void *src, const int32_t *pos, const void *scale
 
 /* Message for the last non-zero return on the calling thread ("" if none). */
 const char *dfa3d_last_error(void);
-
-/* Process-wide launch tunables; results do not depend on them.
- *   "iters"  groups of units each wavefront walks through (default 1)
- *   "vec"    channels per lane in the row gathers: 0 = automatic, 1, 2 or 4 (8: tile kernels only)
- *   "diag"   measurement aid for the backward kernels: bit 0 drops the grad_value updates,
- *            bit 1 the grad_dist updates (results are then incomplete); default 0
- *   "binned" 0 makes dfa3d_fused_backward ignore its workspace (direct atomic kernel); default 1
- *   "tile"   binned backward: tile edge in pixels as ty*100+tx, 0 = automatic
- *   "block"  binned backward: threads per tile workgroup, 256 or 0/512
- *   "pass"   binned backward: points a tile workgroup takes per pass, 128 or 0/256
- *   "chunk"  binned backward: points of one tile handled by one work item, 0 = 4096
- *   "bwd_stage" measurement aid for the binned backward: 0 = every kernel, 1 = the binning kernels
- *            only, 2 = the tile kernel only (on a workspace a stage-1 call has just prepared) */
-int dfa3d_set_tunable(const char *name, int value);
-
-/* Measurement aid: copies `bytes` (a multiple of 16, 16-byte aligned pointers) from src to dst with
- * a plain streaming kernel.  It is the copy of known size that profiler HBM counters are scaled by. */
-int dfa3d_stream_copy(void *dst, const void *src, size_t bytes, void *stream);
 
 /* Library ABI version (bumped when a signature changes). */
 int dfa3d_abi_version(void);

@@ -37,26 +37,27 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     null = ctypes.c_void_p(0)
     one = ctypes.c_void_p(256)          # never dereferenced: validation fails first
     # non-positive dimension
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 0, 10, 8, 32, 16, 2, 5, 4, 8, 0, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 0, 10, 8, 32, 16, 2, 5, 4, 8, 0, None, null)
     assert rc == -1 and b"positive" in L.dfa3d_last_error()
     # unknown dtype
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 7, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 7, None, null)
     assert rc == -1 and b"dtype" in L.dfa3d_last_error()
     # too many levels
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 17, 5, 4, 8, 0, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 17, 5, 4, 8, 0, None, null)
     assert rc == -2 and b"levels" in L.dfa3d_last_error()
     # a batch element beyond 2^30 bytes
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 1 << 20, 8, 64, 16, 2, 5, 4, 8, 0, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 1 << 20, 8, 64, 16, 2, 5, 4, 8, 0, None, null)
     assert rc == -2 and b"2^30" in L.dfa3d_last_error()
     # NULL operand
-    rc = L.dfa3d_fused_forward(null, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 0, null)
+    rc = L.dfa3d_fused_forward(null, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 0, None, null)
     assert rc == -1 and b"NULL" in L.dfa3d_last_error()
     # a distribution for 3 of the 8 heads
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 3, 0, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 3, 0, None, null)
     assert rc == -1 and b"dist_heads" in L.dfa3d_last_error()
-    rc = L.dfa3d_wms_deform_attn_forward(one, one, 4, one, one, 2, one, one, one, 1, 10, 8, 32, 2, 5, 4, 0, null)
+    rc = L.dfa3d_wms_deform_attn_forward(one, one, 4, one, one, 2, one, one, one, 1, 10, 8, 32, 2, 5, 4, 0, None, null)
     assert rc == -1 and b"stride" in L.dfa3d_last_error()
-    rc = L.dfa3d_ms_depth_score_sample_backward(one, one, one, one, one, null, one, null, 0, 1, 10, 8, 16, 2, 5, 4, 0, null)
+    rc = L.dfa3d_ms_depth_score_sample_backward(one, one, one, one, one, null, one, null, 0, 1, 10, 8, 16, 2, 5, 4, 0, None,
+                                                null)
     assert rc == -1 and b"grad_dist" in L.dfa3d_last_error()
     # camera re-batching: dtype, dimensions, pointers
     rc = L.dfa3d_rebatch_gather(one, 0, 16, one, null, one, 1, 6, 8, 16, 4, 2, null)
@@ -67,12 +68,47 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     assert rc == -1 and b"strides" in L.dfa3d_last_error()
     rc = L.dfa3d_rebatch_combine(one, null, null, one, 1, 6, 8, 16, 4, 0, null)
     assert rc == -1 and b"pos is NULL" in L.dfa3d_last_error()
-    assert L.dfa3d_fused_backward_workspace_bytes(6, 30825, 8, 32, 64, 4, 10000, 8, 1, 0) > \
-        L.dfa3d_fused_backward_workspace_bytes(6, 30825, 8, 32, 64, 4, 10000, 8, 8, 0) > 0
-    assert L.dfa3d_fused_backward_workspace_bytes(6, 30825, 8, 32, 64, 4, 10000, 8, 8, 1) == 0    # fp64: direct kernels
-    assert L.dfa3d_set_tunable(b"iters", 0) == -1
-    assert L.dfa3d_set_tunable(b"nope", 1) == -1
-    assert L.dfa3d_set_tunable(b"iters", 1) == 0 and L.dfa3d_set_tunable(b"vec", 0) == 0
+    dims = (6, 30825, 8, 32, 64, 4, 10000, 8)
+    assert L.dfa3d_fused_backward_workspace_bytes(*dims, 1, 0, None) > \
+        L.dfa3d_fused_backward_workspace_bytes(*dims, 8, 0, None) > 0
+    assert L.dfa3d_fused_backward_workspace_bytes(*dims, 8, 1, None) == 0    # fp64: direct kernels
+
+
+def test_launch_options_are_per_call_and_checked():
+    """Launch options travel with each call (no process-wide state): bad values are rejected before anything
+    is launched, `direct` asks for no workspace, and the python context manager restores what it found."""
+    from dfa3D import _lib
+    L = _lib.lib()
+    null, one = ctypes.c_void_p(0), ctypes.c_void_p(256)
+    dims = (1, 10, 8, 32, 16, 2, 5, 4)
+
+    def fwd(**fields):
+        o = _lib.LaunchOptions(**fields)
+        # value is NULL: a call that passes the option checks stops at the operand check
+        return L.dfa3d_fused_forward(null, one, one, one, one, one, one, one, null, *dims, 8, 0, ctypes.pointer(o), null)
+
+    for bad in (dict(iters=-1), dict(iters=65), dict(vec=3), dict(tile=7), dict(tile=6500), dict(block=128),
+                dict(pass_=32), dict(chunk=8), dict(reserved=1)):
+        assert fwd(**bad) == -1 and b"options." in L.dfa3d_last_error(), bad
+    assert fwd(iters=2, vec=4, tile=808, block=256, pass_=128, chunk=1024) == -1 and b"NULL" in L.dfa3d_last_error()
+    big = (6, 30825, 8, 32, 64, 4, 10000, 8)
+    assert L.dfa3d_fused_backward_workspace_bytes(*big, 8, 0, ctypes.pointer(_lib.LaunchOptions(direct=1))) == 0
+    assert L.dfa3d_fused_backward_workspace_bytes(*big, 8, 0, ctypes.pointer(_lib.LaunchOptions(vec=3))) == 0
+    assert L.dfa3d_fused_backward_workspace_bytes(*big, 8, 0, ctypes.pointer(_lib.LaunchOptions(tile=404))) > \
+        L.dfa3d_fused_backward_workspace_bytes(*big, 8, 0, None)            # more, smaller tiles: more counters
+    assert not hasattr(L, "dfa3d_set_tunable") and not hasattr(L, "dfa3d_stream_copy")
+
+    assert _lib.options() is None
+    with _lib.launch_options(tile=404, **{"pass": 128}):
+        with _lib.launch_options(direct=1):
+            o = _lib.options().contents
+            assert (o.tile, o.pass_, o.direct) == (404, 128, 1)
+        o = _lib.options().contents
+        assert (o.tile, o.pass_, o.direct) == (404, 128, 0)
+    assert _lib.options() is None
+    with pytest.raises(TypeError):
+        with _lib.launch_options(nope=1):
+            pass
 
 
 def test_reference_import_paths_and_names():
