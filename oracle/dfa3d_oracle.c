@@ -41,6 +41,17 @@
 #undef REAL
 #undef FN
 
+/* Double arithmetic on the float path's geometry: every sum is (to double precision) the exact sum of the
+ * terms the float instantiation rounds and adds, so |float result - this| is summation and rounding error
+ * alone.  Not a restatement of anything the reference dispatches; same code as the two above. */
+#define REAL double
+#define FN(x) x##_f64g32
+#define DFA3D_ORACLE_FLOAT_GEOMETRY
+#include "dfa3d_oracle_impl.h"
+#undef DFA3D_ORACLE_FLOAT_GEOMETRY
+#undef REAL
+#undef FN
+
 /* Worker threads used by the loops above; returns the previous setting. */
 int dfa3d_oracle_set_threads(int n) {
   int prev = omp_get_max_threads();

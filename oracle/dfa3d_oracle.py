@@ -13,6 +13,7 @@ multi_scale_3ddeformable_attn_function.py:279-303 and :306-352).
 All arguments are contiguous CPU ``torch`` tensors, float32 or float64
 (shapes/level starts int64), the two types the reference dispatches.
 """
+import contextlib
 import ctypes
 import os
 import subprocess
@@ -51,11 +52,26 @@ def get_threads():
     return lib().dfa3d_oracle_get_threads()
 
 
+_float_geometry = False
+
+
+@contextlib.contextmanager
+def float_geometry():
+    """Inside the block, float64 calls use the float32 path's pixel coordinates (the locations must be float32
+    values held in float64): their sums are then the exact sums of the terms the float32 path adds up."""
+    global _float_geometry
+    saved, _float_geometry = _float_geometry, True
+    try:
+        yield
+    finally:
+        _float_geometry = saved
+
+
 def _suffix(t):
     if t.dtype == torch.float32:
         return "f32"
     if t.dtype == torch.float64:
-        return "f64"
+        return "f64g32" if _float_geometry else "f64"
     raise TypeError(f"oracle handles float32/float64 only, got {t.dtype}")
 
 

@@ -1,8 +1,10 @@
 /*
  * TEST INFRASTRUCTURE ONLY - scalar CPU restatement of the DFA3D operator, one
- * precision per inclusion.  Included twice by dfa3d_oracle.c with
+ * precision per inclusion.  Included by dfa3d_oracle.c with
  *   REAL   = float  / double
  *   FN(x)  = x##_f32 / x##_f64
+ * and a third time as x##_f64g32: double arithmetic on the float path's pixel
+ * coordinates (DFA3D_ORACLE_FLOAT_GEOMETRY), the yardstick for float summation error.
  *
  * Every routine states the reference lines it restates.  Paths are relative to
  * the reference checkout; "ms.cuh" is
@@ -26,8 +28,16 @@ static const int FN(k_visit)[4] = {0, 1, 3, 2};
 /* Pixel coordinate of a normalised location (ms.cuh:133-135, wms.cuh:286-287):
  * float product, then "- 0.5" with a double literal, rounded back to REAL. */
 static inline REAL FN(to_pixel)(REAL loc, int size) {
+#ifdef DFA3D_ORACLE_FLOAT_GEOMETRY
+  /* the float kernels' pixel coordinate (locations that are float values held in doubles), so that the
+   * double sums of this instantiation are the exact sums of the terms the float path adds up */
+  const float prod = (float)loc * size;
+  const float imf = (float)(prod - 0.5);
+  return imf;
+#else
   const REAL im = loc * size - 0.5;
   return im;
+#endif
 }
 
 /* floor as the reference takes it: floorf() on every scalar type, so a double

@@ -272,3 +272,27 @@ def test_thread_count_does_not_change_results(oracle):
         oracle.set_threads(prev)
     for x, y in zip(a + ga, b + gb):
         assert torch.equal(x, y)
+
+
+def test_float_geometry_instantiation_tracks_both_precisions(oracle):
+    """The third instantiation of the checker (float64 arithmetic on the float32 path's pixel coordinates, the
+    yardstick for float32 summation error in the GPU tests) is the same code as the other two: on float32
+    inputs it agrees with the float64 instantiation up to what a float32 pixel coordinate is worth, and with
+    the float32 instantiation up to float32 rounding of the sums."""
+    t = tiny_case(77, B=2, C=8, M=3, Q=40, P=4, D=6, levels=((90, 120), (7, 9)), dtype=torch.float32)
+    args32 = (t["value"], t["dist"], t["shapes3"], t["lsi"], t["loc"], t["attn"])
+    args64 = tuple(a.double() if a.is_floating_point() else a for a in args32)
+
+    def run(args, go):
+        out, score = oracle.dfa3d_forward(*args)
+        return (out, score) + tuple(oracle.dfa3d_backward(*args, score, go))
+
+    r32 = run(args32, t["grad_out"])
+    r64 = run(args64, t["grad_out"].double())
+    with oracle.float_geometry():
+        rg = run(args64, t["grad_out"].double())
+    for a, b, c in zip(r32, r64, rg):
+        assert c.dtype == torch.float64
+        torch.testing.assert_close(c, b, rtol=1e-4, atol=1e-4)                 # coordinates differ by <= 120 * 2^-24
+        torch.testing.assert_close(c, a.double(), rtol=1e-5, atol=2e-6)        # sums differ by float32 rounding
+    assert not torch.equal(rg[2], r64[2])                                      # and it is not the plain float64 path
