@@ -2,7 +2,7 @@
 """Benchmark of the DFA3D operator on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload base|small|unit|dense|base_bf16|unittest]
-    python bench.py --micro                      yardsticks of the machine (copy, bare gathers, LDS atomics, XCD map)
+    python bench.py --micro [xcd]                yardsticks of the machine (copy, bare gathers, LDS atomics, XCD map)
     python bench.py --summarize NAME DIR [DIR..] tables from rocprofv3 output directories -> profiles/NAME.txt
 
 A step is one forward + backward of the one-stage autograd Function
@@ -57,7 +57,8 @@ def parse():
                     help="skip the timings of the two-stage, shared-distribution and plain-attention entry points")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="launch option for every library call (%s)" % ", ".join(OPTION_NAMES))
-    ap.add_argument("--micro", action="store_true", help="run the yardstick kernels instead of the operator")
+    ap.add_argument("--micro", nargs="?", const="all", choices=("all", "xcd"),
+                    help="run the yardstick kernels instead of the operator (xcd: only the workgroup -> XCD map)")
     ap.add_argument("--summarize", nargs="+", metavar=("NAME", "DIR"),
                     help="write profiles/NAME.txt (and profiles/hbm_traffic.json) from rocprofv3 output directories")
     ap.add_argument("--summarize-command", action="append", default=[],
@@ -124,7 +125,7 @@ def copy_bandwidth(torch, mib=1024, reps=5):
     return 2 * n / (best * 1e-3) / 1e9
 
 
-def micro():
+def micro(sections="all"):
     """Yardsticks: what the machine does for the bare access patterns of the kernels."""
     import torch
     m = measure_lib()
@@ -152,6 +153,9 @@ def micro():
                          "xcd_of_block_mod_8": hist.argmax(1).tolist(), "xcds_seen": int(x.unique().numel())})
         maps[f"{blocks}x{threads}"] = rows
     out["xcd_map"] = maps
+    if sections == "xcd":
+        print(json.dumps(out))
+        return
 
     # random whole-row gathers (the value-row gathers of the forward) against the footprint they are drawn from
     src = torch.zeros(1 << 30, dtype=torch.uint8, device=dev)
@@ -414,7 +418,7 @@ def main():
         print("bench.py: no GPU visible; the HIP kernels are the product and there is no fallback", file=sys.stderr)
         sys.exit(3)
     if a.micro:
-        micro()
+        micro(a.micro)
         return
     L_ = _lib.lib()
     user_options = {}
