@@ -2,6 +2,7 @@
 // Errors are returned, never printed-and-ignored (the reference's launchers only printf a failed
 // launch: DFA3D/dfa3D/ops/csrc/cuda/wms_deform_attn_cuda.cu:45-48).
 #include <atomic>
+#include <mutex>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -296,6 +297,67 @@ int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *sha
     if (e != hipErrorNotSupported) return hip_result(e, fn);
   }
   return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
+}
+
+// ---------------------------------------------------------------------------------------
+// dfa3d_fused_backward_static: the binned backward on a scratch buffer that is part of the library's
+// code object instead of memory the caller allocates.  Each GPU holds its own copy of the array at its
+// own address; host code must not use the array's name as a pointer (it is a host-side stand-in), so the
+// device address is asked for once per device and kept.
+// ---------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[DFA3D_STATIC_SCRATCH_BYTES];
+
+static constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void *g_scratch_ptr[kMaxDevices];          // device address of `scratch` on each GPU, nullptr = not asked yet
+
+// Device address of this GPU's copy of `scratch` (the current device's), looked up on first use.
+static int static_scratch(const char *fn, void **out) {
+  int dev = -1;
+  if (hipError_t e = hipGetDevice(&dev)) return hip_result(e, fn);
+  if (dev < 0 || dev >= kMaxDevices) return fail(DFA3D_ERANGE, "%s: device ordinal %d not supported", fn, dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *p = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) return hip_result(e, fn);
+    if (p == nullptr || ((uintptr_t)p & 255) != 0) return fail(DFA3D_EINVAL, "%s: bad address for the static scratch", fn);
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+size_t dfa3d_static_scratch_bytes(void) { return DFA3D_STATIC_SCRATCH_BYTES; }
+
+int dfa3d_fused_backward_static(const void *value, const void *dist, const int64_t *shapes3,
+                                const int64_t *level_start, const void *loc3, const void *attn,
+                                const void *grad_out, const void *grad_score_in, const void *grad_weight_update,
+                                void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn, int B, int S,
+                                int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype,
+                                const dfa3d_launch_options *opts, void *stream) {
+  const char *fn = "dfa3d_fused_backward_static";
+  dfa3d_launch_options o;
+  if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
+  if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
+  if (int rc = check_opts(fn, opts, &o)) return rc;
+  if (dist_heads != M && dist_heads != 1) return fail(DFA3D_EINVAL, "%s: dist_heads must be M or 1", fn);
+  REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
+  REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
+  REQUIRE_PTR(fn, grad_dist); REQUIRE_PTR(fn, grad_loc3); REQUIRE_PTR(fn, grad_attn);
+  const dfa3d::BwdArgs a = fused_bwd_args(value, dist, shapes3, level_start, loc3, attn, grad_out, grad_score_in,
+                                          grad_weight_update, grad_value, grad_dist, grad_loc3, grad_attn, B, S, M, C,
+                                          D, L, Q, P, dist_heads, o);
+  const size_t need = o.direct ? 0 : dfa3d::binned_backward_workspace_bytes(a, 0, dtype);
+  if (need > DFA3D_STATIC_SCRATCH_BYTES)
+    return fail(DFA3D_ERANGE, "%s: these dimensions need %zu bytes of scratch, the static buffer holds %zu; use "
+                "dfa3d_fused_backward with a workspace", fn, need, (size_t)DFA3D_STATIC_SCRATCH_BYTES);
+  if (need > 0) {
+    void *ws = nullptr;
+    if (int rc = static_scratch(fn, &ws)) return rc;
+    const hipError_t e = dfa3d::launch_backward_binned(a, dtype, ws, DFA3D_STATIC_SCRATCH_BYTES, (hipStream_t)stream);
+    if (e != hipErrorNotSupported) return hip_result(e, fn);
+  }
+  return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);   // no scratch needed at all
 }
 
 static int check_rebatch(const char *fn, int bs, int cams, int max_len, int Nq, int E, int dtype) {

@@ -38,6 +38,7 @@ SIGNATURES = {
     + _DIMS7 + [_I, _O, _P],
     "dfa3d_fused_forward": [_P] * 9 + _DIMS8 + [_I, _I, _O, _P],
     "dfa3d_fused_backward": [_P] * 14 + [ctypes.c_size_t] + _DIMS8 + [_I, _I, _O, _P],
+    "dfa3d_fused_backward_static": [_P] * 13 + _DIMS8 + [_I, _I, _O, _P],
     "dfa3d_rebatch_gather": [_P, ctypes.c_longlong, ctypes.c_longlong, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "dfa3d_rebatch_combine": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "dfa3d_abi_version": [],
@@ -65,6 +66,8 @@ def lib():
             fn = getattr(handle, name)
             fn.argtypes = dims + [_I, _O]
             fn.restype = ctypes.c_size_t
+        handle.dfa3d_static_scratch_bytes.argtypes = []
+        handle.dfa3d_static_scratch_bytes.restype = ctypes.c_size_t
         handle.dfa3d_last_error.argtypes = []
         handle.dfa3d_last_error.restype = ctypes.c_char_p
         if handle.dfa3d_abi_version() != ABI_VERSION:

@@ -164,6 +164,27 @@ int dfa3d_fused_backward(
 size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads,
                                             int dtype, const dfa3d_launch_options *opts);
 
+/* dfa3d_fused_backward for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and
+ * results as dfa3d_fused_backward, without the workspace: the scratch memory of the binned kernels is a static
+ * array of DFA3D_STATIC_SCRATCH_BYTES inside the library's code object, which every GPU the library runs on
+ * holds until the process ends.  The call allocates and frees nothing.  Dimensions whose
+ * dfa3d_fused_backward_workspace_bytes exceeds that size are rejected with DFA3D_ERANGE (at the BEVFormer-small
+ * shape, 1.5 M sampling points, the kernels want 29.8 MiB); dimensions the binned path does not apply to
+ * (workspace size 0, e.g. DFA3D_F64) run on the direct kernels, which need no scratch.
+ * Every call on one GPU uses that GPU's one array: calls that overlap in time on the same GPU (two streams, two
+ * threads) race and give wrong gradients; calls on one stream, or otherwise ordered, are safe, and nothing has
+ * to be cleared between them. */
+#define DFA3D_STATIC_SCRATCH_BYTES (32u << 20)
+int dfa3d_fused_backward_static(
+    const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
+    const void *loc3, const void *attn, const void *grad_out, const void *grad_score_in,
+    const void *grad_weight_update,
+    void *grad_value, void *grad_dist, void *grad_loc3, void *grad_attn,
+    int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype,
+    const dfa3d_launch_options *opts, void *stream);
+size_t dfa3d_static_scratch_bytes(void);
+
 /* Camera re-batching around the operator, as DFA3D-BEVFormer's spatial cross-attention does it in python
  * loops over batch x cameras
  * (BEVFormer_DFA3D/projects/mmdet3d_plugin/bevformer/modules/spatial_cross_attention.py:716-722, 741-748).
