@@ -104,18 +104,26 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
           const int l = lp / P;
           const size_t gp = ((size_t)(b * (size_t)Q + q) * M + m) * ws.LP + lp;   // global point index
           const A *pl = loc + gp * loc_stride;
-          const A x = pl[0], y = pl[1];
-          const A a = attn[gp];
+          // locations, weights and scores pass through once: non-temporal, so that they do not push the value
+          // rows and distributions that the gathers keep coming back to out of the L2
+          const A x = __builtin_nontemporal_load(pl), y = __builtin_nontemporal_load(pl + 1);
+          const A a = __builtin_nontemporal_load(attn + gp);
           const Point2D<A> g = locate_2d<A>(x, y, tab.H[l], tab.W[l], tab.start[l]);
           A sc[4];
           if (FUSED) {
             A lo[4], hi[4];
-            const DepthTap<A> tap = locate_depth<A>(pl[2], tab.Dd[l]);
+            const DepthTap<A> tap = locate_depth<A>(__builtin_nontemporal_load(pl + 2), tab.Dd[l]);
             corner_scores<T, A>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
             if (score_out != nullptr && pass == 0) {
               T *so = score_out + gp * 4;
+              if constexpr (sizeof(T) == 4) {                     // one 16-byte store
+                typedef float f4 __attribute__((ext_vector_type(4)));
+                f4 v4 = {(float)sc[0], (float)sc[1], (float)sc[2], (float)sc[3]};
+                __builtin_nontemporal_store(v4, reinterpret_cast<f4 *>(so));
+              } else {
 #pragma unroll
-              for (int k = 0; k < 4; ++k) Elem<T>::st(so + k, sc[k]);
+                for (int k = 0; k < 4; ++k) Elem<T>::st(so + k, sc[k]);
+              }
             }
             wu = a * ((sc[0] + sc[1] + sc[2] + sc[3]) * (A)0.25);
           } else {

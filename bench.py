@@ -216,39 +216,47 @@ def short_name(n):
 
 
 def summarize(name, dirs, commands):
-    """Per-kernel tables from rocprofv3's rocpd databases (kernel durations; counters per dispatch) as text under
-    profiles/, and the HBM-side bytes of the operator's kernels (FETCH_SIZE / WRITE_SIZE, each scaled by what the
-    same counter reads for the yardstick copy of known size in the same run) into profiles/hbm_traffic.json."""
+    """Per-kernel tables from rocprofv3's rocpd databases (kernel durations; counters per dispatch, averaged) as
+    text under profiles/, and the HBM-side bytes of the operator's kernels (FETCH_SIZE / WRITE_SIZE, each scaled
+    by what the same counter reads for the yardstick copy of known size in the same run) into
+    profiles/hbm_traffic.json."""
     import sqlite3
     lines = [f"# {c}" for c in commands]
     scale, raw, workload = {}, {}, None
+    cols = ("fwd_attention_kernel", "tile_backward_kernel", "bin_points_kernel<0>", "bin_points_kernel<1>",
+            "stream_copy_kernel")
     for d in dirs:
         for db in sorted(glob.glob(os.path.join(d, "**", "*.db"), recursive=True)):
             c = sqlite3.connect(db)
-            rows = c.execute("select name, count(*), avg(end-start), min(end-start), max(end-start), sum(end-start) "
-                             "from kernels group by name order by 6 desc").fetchall()
-            tot = sum(r[5] for r in rows) or 1
-            lines += ["", f"## {os.path.relpath(db, ROOT)}: kernel durations",
-                      f"{'kernel':94s} {'calls':>5s} {'avg_us':>10s} {'min_us':>10s} {'max_us':>10s} {'pct':>6s}"]
-            for n, k, a, mi, ma, s in rows[:16]:
-                lines.append(f"{short_name(n):94s} {k:5d} {a / 1e3:10.1f} {mi / 1e3:10.1f} {ma / 1e3:10.1f} {100 * s / tot:6.1f}")
             try:
-                rows = c.execute("select kernel_name, counter_name, count(*), avg(value), min(value), max(value) from "
-                                 "counters_collection group by kernel_name, counter_name order by 1, 2").fetchall()
+                rows = c.execute("select kernel_name, counter_name, count(*), avg(value) from counters_collection "
+                                 "group by kernel_name, counter_name order by 2, 1").fetchall()
             except sqlite3.Error:
                 rows = []
-            if rows:
-                lines += ["", f"## {os.path.relpath(db, ROOT)}: counters per dispatch (raw)",
-                          f"{'kernel':94s} {'counter':>22s} {'n':>4s} {'avg':>16s} {'min':>16s} {'max':>16s}"]
-            for n, cn, k, a, mi, ma in rows:
-                if "dfa3d" not in n and "stream_copy" not in n:
-                    continue
-                lines.append(f"{short_name(n):94s} {cn:>22s} {k:4d} {a:16.1f} {mi:16.1f} {ma:16.1f}")
-                if "stream_copy_kernel" in n and cn in ("FETCH_SIZE", "WRITE_SIZE"):
-                    scale[cn] = a
-                for frag, key in KERNEL_KEYS:
-                    if frag in n and cn in ("FETCH_SIZE", "WRITE_SIZE"):
-                        raw.setdefault(key, {})[cn] = a
+            rel = os.path.relpath(db, ROOT)
+            if not rows:
+                k = c.execute("select name, count(*), avg(end-start), min(end-start), max(end-start), sum(end-start) "
+                              "from kernels group by name order by 6 desc").fetchall()
+                tot = sum(r[5] for r in k) or 1
+                lines += ["", f"## {rel}: kernel durations",
+                          f"{'kernel':64s} {'calls':>5s} {'avg_us':>9s} {'min_us':>9s} {'max_us':>9s} {'pct':>5s}"]
+                for n, cnt, a, mi, ma, sm in k[:12]:
+                    lines.append(f"{short_name(n)[:64]:64s} {cnt:5d} {a / 1e3:9.1f} {mi / 1e3:9.1f} {ma / 1e3:9.1f} {100 * sm / tot:5.1f}")
+            else:
+                table = {}
+                for n, cn, cnt, a in rows:
+                    for col in cols:
+                        if col in n:
+                            table.setdefault(cn, {})[col] = a
+                    if "stream_copy_kernel" in n and cn in ("FETCH_SIZE", "WRITE_SIZE"):
+                        scale[cn] = a
+                    for frag, key in KERNEL_KEYS:
+                        if frag in n and cn in ("FETCH_SIZE", "WRITE_SIZE"):
+                            raw.setdefault(key, {})[cn] = a
+                lines += ["", f"## {rel}: counters, average per dispatch (raw)",
+                          f"{'counter':36s} " + " ".join(f"{col[:20]:>20s}" for col in cols)]
+                for cn in sorted(table):
+                    lines.append(f"{cn:36s} " + " ".join(f"{table[cn].get(col, float('nan')):20.1f}" for col in cols))
             c.close()
     mib = None
     for cmd in commands:
@@ -263,9 +271,9 @@ def summarize(name, dirs, commands):
     traffic = {}
     if copy_kib and "FETCH_SIZE" in scale and "WRITE_SIZE" in scale:
         f_scale, w_scale = copy_kib / scale["FETCH_SIZE"], copy_kib / scale["WRITE_SIZE"]
-        lines += ["", f"## HBM-side bytes per launch: counter (KiB) x 1024 x scale factor; the yardstick copy moves "
-                      f"{copy_kib} KiB each way, FETCH_SIZE reads {scale['FETCH_SIZE']:.0f} for it (factor {f_scale:.3f}), "
-                      f"WRITE_SIZE {scale['WRITE_SIZE']:.0f} (factor {w_scale:.3f})"]
+        lines += ["", f"## HBM-side bytes per launch = counter (KiB) x 1024 x scale factor.  The yardstick copy moves "
+                      f"{copy_kib} KiB each way;", f"## FETCH_SIZE reads {scale['FETCH_SIZE']:.0f} for it (factor "
+                      f"{f_scale:.3f}), WRITE_SIZE {scale['WRITE_SIZE']:.0f} (factor {w_scale:.3f})"]
         for key, v in raw.items():
             if "FETCH_SIZE" in v and "WRITE_SIZE" in v:
                 fb, wb = v["FETCH_SIZE"] * 1024 * f_scale, v["WRITE_SIZE"] * 1024 * w_scale
