@@ -72,7 +72,8 @@ void apply_opts(dfa3d::BwdArgs &a, const dfa3d_launch_options &o) {
 // Dimension checks shared by every entry point.  `width` is the per-head row length (C or D).
 int check_dims(const char *fn, int B, int S, int M, int width, int L, int Q, int P, int dtype) {
   if (dtype != DFA3D_F32 && dtype != DFA3D_F64 && dtype != DFA3D_BF16)
-    return fail(DFA3D_EINVAL, "%s: unknown dtype %d", fn, dtype);
+    return fail(DFA3D_EINVAL, "%s: unknown dtype %d%s", fn, dtype,
+                dtype == DFA3D_BF16G ? " (DFA3D_BF16G is for the dfa3d_fused_backward calls only)" : "");
   if (B <= 0 || S <= 0 || M <= 0 || width <= 0 || L <= 0 || Q <= 0 || P <= 0)
     return fail(DFA3D_EINVAL, "%s: dimensions must be positive (B=%d S=%d M=%d C|D=%d L=%d Q=%d P=%d)", fn, B, S, M,
                 width, L, Q, P);
@@ -264,13 +265,16 @@ size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, i
                                             int dtype, const dfa3d_launch_options *opts) {
   const char *fn = "dfa3d_fused_backward_workspace_bytes";
   dfa3d_launch_options o;
+  const bool g16 = dtype == DFA3D_BF16G;
+  if (g16) dtype = DFA3D_BF16;
   if (check_dims(fn, B, S, M, C, L, Q, P, dtype) || check_dims(fn, B, S, M, D, L, Q, P, dtype) ||
       check_opts(fn, opts, &o))
     return 0;
   if (o.direct) return 0;
-  const dfa3d::BwdArgs a = fused_bwd_args(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
-                                          nullptr, nullptr, nullptr, nullptr, nullptr, B, S, M, C, D, L, Q, P,
-                                          dist_heads == 1 ? 1 : M, o);
+  dfa3d::BwdArgs a = fused_bwd_args(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                                    nullptr, nullptr, nullptr, nullptr, nullptr, B, S, M, C, D, L, Q, P,
+                                    dist_heads == 1 ? 1 : M, o);
+  a.grad_bf16 = g16;
   return dfa3d::binned_backward_workspace_bytes(a, 0, dtype);
 }
 
@@ -282,6 +286,8 @@ int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *sha
                          const dfa3d_launch_options *opts, void *stream) {
   const char *fn = "dfa3d_fused_backward";
   dfa3d_launch_options o;
+  const bool g16 = dtype == DFA3D_BF16G;
+  if (g16) dtype = DFA3D_BF16;
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
   if (int rc = check_opts(fn, opts, &o)) return rc;
@@ -289,13 +295,17 @@ int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *sha
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
   REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
   REQUIRE_PTR(fn, grad_dist); REQUIRE_PTR(fn, grad_loc3); REQUIRE_PTR(fn, grad_attn);
-  const dfa3d::BwdArgs a = fused_bwd_args(value, dist, shapes3, level_start, loc3, attn, grad_out, grad_score_in,
-                                          grad_weight_update, grad_value, grad_dist, grad_loc3, grad_attn, B, S, M, C,
-                                          D, L, Q, P, dist_heads, o);
+  dfa3d::BwdArgs a = fused_bwd_args(value, dist, shapes3, level_start, loc3, attn, grad_out, grad_score_in,
+                                    grad_weight_update, grad_value, grad_dist, grad_loc3, grad_attn, B, S, M, C,
+                                    D, L, Q, P, dist_heads, o);
+  a.grad_bf16 = g16;
   if (workspace != nullptr && !o.direct) {
     const hipError_t e = dfa3d::launch_backward_binned(a, dtype, workspace, workspace_bytes, (hipStream_t)stream);
     if (e != hipErrorNotSupported) return hip_result(e, fn);
   }
+  if (g16) return fail(DFA3D_EINVAL, "%s: DFA3D_BF16G (bfloat16 gradients) runs on the binned kernels only: pass a "
+                       "workspace of dfa3d_fused_backward_workspace_bytes(..., DFA3D_BF16G, ...) bytes (0 = not offered "
+                       "for these dimensions: use DFA3D_BF16 with float gradients)", fn);
   return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
 }
 
@@ -337,6 +347,8 @@ int dfa3d_fused_backward_static(const void *value, const void *dist, const int64
                                 const dfa3d_launch_options *opts, void *stream) {
   const char *fn = "dfa3d_fused_backward_static";
   dfa3d_launch_options o;
+  const bool g16 = dtype == DFA3D_BF16G;
+  if (g16) dtype = DFA3D_BF16;
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
   if (int rc = check_opts(fn, opts, &o)) return rc;
@@ -344,9 +356,10 @@ int dfa3d_fused_backward_static(const void *value, const void *dist, const int64
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
   REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
   REQUIRE_PTR(fn, grad_dist); REQUIRE_PTR(fn, grad_loc3); REQUIRE_PTR(fn, grad_attn);
-  const dfa3d::BwdArgs a = fused_bwd_args(value, dist, shapes3, level_start, loc3, attn, grad_out, grad_score_in,
-                                          grad_weight_update, grad_value, grad_dist, grad_loc3, grad_attn, B, S, M, C,
-                                          D, L, Q, P, dist_heads, o);
+  dfa3d::BwdArgs a = fused_bwd_args(value, dist, shapes3, level_start, loc3, attn, grad_out, grad_score_in,
+                                    grad_weight_update, grad_value, grad_dist, grad_loc3, grad_attn, B, S, M, C,
+                                    D, L, Q, P, dist_heads, o);
+  a.grad_bf16 = g16;
   const size_t need = o.direct ? 0 : dfa3d::binned_backward_workspace_bytes(a, 0, dtype);
   if (need > DFA3D_STATIC_SCRATCH_BYTES)
     return fail(DFA3D_ERANGE, "%s: these dimensions need %zu bytes of scratch, the static buffer holds %zu; use "
@@ -357,6 +370,7 @@ int dfa3d_fused_backward_static(const void *value, const void *dist, const int64
     const hipError_t e = dfa3d::launch_backward_binned(a, dtype, ws, DFA3D_STATIC_SCRATCH_BYTES, (hipStream_t)stream);
     if (e != hipErrorNotSupported) return hip_result(e, fn);
   }
+  if (g16) return fail(DFA3D_EINVAL, "%s: DFA3D_BF16G is not offered for these dimensions", fn);
   return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);   // no scratch needed at all
 }
 

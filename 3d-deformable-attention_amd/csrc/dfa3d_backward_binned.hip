@@ -431,9 +431,10 @@ template <typename T, int VEC, int LPR, bool FUSED>
 __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
     BinWorkspace ws, const T *__restrict__ value, const T *__restrict__ dist, const T *__restrict__ score_in,
     const T *__restrict__ grad_out, const T *__restrict__ grad_score_in,
-    float *__restrict__ grad_value, float *__restrict__ grad_dist, float *__restrict__ grad_loc, int gl_stride,
+    void *__restrict__ grad_value, void *__restrict__ grad_dist, float *__restrict__ grad_loc, int gl_stride,
     float *__restrict__ grad_attn, float *__restrict__ grad_score_out, const float *__restrict__ grad_wu, int Md,
-    int Mg, int B, int S, int M, int C, int D, int L, int Q, int P, int PP, int diag) {
+    int Mg, int B, int S, int M, int C, int D, int L, int Q, int P, int PP, int grad16, int diag) {
+  // grad16: bit 0 = grad_value is bfloat16, bit 1 = grad_dist is bfloat16 (else float)
   // Md: heads stored in dist (M, or 1 = shared by all heads); Mg: heads of the grad_dist buffer written here
   constexpr int RPI = kWave / LPR;                  // row groups per wavefront
   extern __shared__ __align__(16) float smem[];
@@ -811,9 +812,10 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
     __syncthreads();                                     // the tile is complete
 
     // ---------------- flush the tile (and leave it zeroed for the next item) ----------------
-    float *gvalue_b = grad_value + (size_t)b * S * M * C;
+    const bool gv16 = (grad16 & 1) != 0, gd16 = (grad16 & 2) != 0;          // uniform
     const int mg = Mg == 1 ? 0 : m;
-    float *gdist_b = FUSED ? grad_dist + (size_t)b * S * Mg * D : nullptr;
+    char *gvalue_b = static_cast<char *>(grad_value) + (size_t)b * S * M * C * (gv16 ? 2 : 4);
+    char *gdist_b = FUSED ? static_cast<char *>(grad_dist) + (size_t)b * S * Mg * D * (gd16 ? 2 : 4) : nullptr;
     const rsrc_t gvalue_r = make_rsrc(gvalue_b, (size_t)S * M * C * sizeof(float));
     const rsrc_t gdist_r = make_rsrc(gdist_b, FUSED ? (size_t)S * Mg * D * sizeof(float) : 0);
     // Rows 1..TY-1 x 1..TX-1 of the tile belong to no neighbour's halo; when this item holds all the
@@ -821,6 +823,28 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
     // (grad_value and grad_dist are zero on entry).
     const bool sole = chunks_here == 1;
     const bool sole_d = sole && Mg == M;                 // a gradient shared by the heads collects from all of them
+    // four consecutive elements at element index `e` of a batch slice: stored, or added atomically
+    auto put4 = [&](char *base, rsrc_t r, bool is16, uint32_t e, const float4 &val, bool store, bool every) {
+      if (!is16) {
+        float *fb = reinterpret_cast<float *>(base);
+        if (store) {
+          *reinterpret_cast<float4 *>(fb + e) = val;                              // zeros too: full lines
+        } else {
+          if (every || val.x != 0) scatter_add(r, fb, e * 4, val.x);
+          if (every || val.y != 0) scatter_add(r, fb, e * 4 + 4, val.y);
+          if (every || val.z != 0) scatter_add(r, fb, e * 4 + 8, val.z);
+          if (every || val.w != 0) scatter_add(r, fb, e * 4 + 12, val.w);
+        }
+      } else {
+        char *dst = base + (size_t)e * 2;
+        if (store) {
+          *reinterpret_cast<uint2 *>(dst) = make_uint2(pack_bf16x2(val.x, val.y), pack_bf16x2(val.z, val.w));
+        } else {
+          if (val.x != 0 || val.y != 0) atomic_add_bf16x2(dst, val.x, val.y);
+          if (val.z != 0 || val.w != 0) atomic_add_bf16x2(dst + 4, val.z, val.w);
+        }
+      }
+    };
     if (((C | D) & 3) == 0) {
       // four floats per lane: whole 128-byte lines leave each row group at once
       const int c4n = C >> 2, d4n = D >> 2;
@@ -832,15 +856,9 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const int ry = r / TW, rx = r - ry * TW;
         const int y = y0 + ry, x = x0 + rx;
         if (y < H && x < W && !DFA3D_DIAG(diag, 4)) {
-          const uint32_t off = (uint32_t)((((start + y * W + x) * M + m) * C + c) * 4);
-          if (sole && ry >= 1 && ry < TY && rx >= 1 && rx < TX) {
-            *reinterpret_cast<float4 *>(gvalue_b + (off >> 2)) = val;          // zeros too: full lines
-          } else if (nz) {
-            scatter_add(gvalue_r, gvalue_b, off, val.x);
-            scatter_add(gvalue_r, gvalue_b, off + 4, val.y);
-            scatter_add(gvalue_r, gvalue_b, off + 8, val.z);
-            scatter_add(gvalue_r, gvalue_b, off + 12, val.w);
-          }
+          const uint32_t e = (uint32_t)(((start + y * W + x) * M + m) * C + c);
+          const bool store = sole && ry >= 1 && ry < TY && rx >= 1 && rx < TX;
+          if (store || nz) put4(gvalue_b, gvalue_r, gv16, e, val, store, true);
         }
       }
       for (int i = tid; i < R * d4n; i += n_thr) {
@@ -851,38 +869,35 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const int ry = r / TW, rx = r - ry * TW;
         const int y = y0 + ry, x = x0 + rx;
         if (y < H && x < W && !DFA3D_DIAG(diag, 4)) {
-          const uint32_t off = (uint32_t)((((start + y * W + x) * Mg + mg) * D + d) * 4);
-          if (sole_d && ry >= 1 && ry < TY && rx >= 1 && rx < TX) {
-            *reinterpret_cast<float4 *>(gdist_b + (off >> 2)) = val;
-          } else if (nz) {
-            if (val.x != 0) scatter_add(gdist_r, gdist_b, off, val.x);
-            if (val.y != 0) scatter_add(gdist_r, gdist_b, off + 4, val.y);
-            if (val.z != 0) scatter_add(gdist_r, gdist_b, off + 8, val.z);
-            if (val.w != 0) scatter_add(gdist_r, gdist_b, off + 12, val.w);
-          }
+          const uint32_t e = (uint32_t)(((start + y * W + x) * Mg + mg) * D + d);
+          const bool store = sole_d && ry >= 1 && ry < TY && rx >= 1 && rx < TX;
+          if (store || nz) put4(gdist_b, gdist_r, gd16, e, val, store, false);
         }
       }
-    } else {
-    for (int i = tid; i < R * C; i += n_thr) {
-      const float val = gv[i];
-      if (val != 0) {
-        gv[i] = 0;
-        const int r = i / C, c = i - r * C;
-        const int ry = r / TW, rx = r % TW;
-        const int y = y0 + ry, x = x0 + rx;
-        if (y < H && x < W && !DFA3D_DIAG(diag, 4)) scatter_add(gvalue_r, gvalue_b, (uint32_t)((((start + y * W + x) * M + m) * C + c) * 4), val);
+    } else {                                                    // float gradients only (the launcher sees to it)
+      float *gvalue_f = reinterpret_cast<float *>(gvalue_b), *gdist_f = reinterpret_cast<float *>(gdist_b);
+      for (int i = tid; i < R * C; i += n_thr) {
+        const float val = gv[i];
+        if (val != 0) {
+          gv[i] = 0;
+          const int r = i / C, c = i - r * C;
+          const int ry = r / TW, rx = r % TW;
+          const int y = y0 + ry, x = x0 + rx;
+          if (y < H && x < W && !DFA3D_DIAG(diag, 4))
+            scatter_add(gvalue_r, gvalue_f, (uint32_t)((((start + y * W + x) * M + m) * C + c) * 4), val);
+        }
       }
-    }
-    for (int i = tid; i < R * D; i += n_thr) {
-      const float val = gd[i];
-      if (val != 0) {
-        gd[i] = 0;
-        const int r = i / D, d = i - r * D;
-        const int ry = r / TW, rx = r % TW;
-        const int y = y0 + ry, x = x0 + rx;
-        if (y < H && x < W && !DFA3D_DIAG(diag, 4)) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * Mg + mg) * D + d) * 4), val);
+      for (int i = tid; i < R * D; i += n_thr) {
+        const float val = gd[i];
+        if (val != 0) {
+          gd[i] = 0;
+          const int r = i / D, d = i - r * D;
+          const int ry = r / TW, rx = r % TW;
+          const int y = y0 + ry, x = x0 + rx;
+          if (y < H && x < W && !DFA3D_DIAG(diag, 4))
+            scatter_add(gdist_r, gdist_f, (uint32_t)((((start + y * W + x) * Mg + mg) * D + d) * 4), val);
+        }
       }
-    }
     }
     TT_MARK(6);
   }
@@ -1026,9 +1041,10 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(float4 *__restrict__ dst
     dst[i] = make_float4(0, 0, 0, 0);
 }
 
-// dst[r, :] = sum over heads m of src[r, m, :], rows of D floats, heads in order
-__global__ __launch_bounds__(256) void head_sum_kernel(const float *__restrict__ src, float *__restrict__ dst,
-                                                       size_t rows, int M, int D) {
+// dst[r, :] = sum over heads m of src[r, m, :], rows of D floats, heads in order; dst is float, or bfloat16
+// when dst16 is set (then D is a multiple of 4)
+__global__ __launch_bounds__(256) void head_sum_kernel(const float *__restrict__ src, void *__restrict__ dst,
+                                                       size_t rows, int M, int D, int dst16) {
   if ((D & 3) == 0) {
     const int d4 = D >> 2;
     const size_t n = rows * d4;
@@ -1040,7 +1056,11 @@ __global__ __launch_bounds__(256) void head_sum_kernel(const float *__restrict__
         const float4 t = *reinterpret_cast<const float4 *>(src + (r * M + m) * D + d);
         acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
       }
-      *reinterpret_cast<float4 *>(dst + r * D + d) = acc;
+      if (dst16)
+        *reinterpret_cast<uint2 *>(static_cast<char *>(dst) + (r * D + d) * 2) =
+            make_uint2(pack_bf16x2(acc.x, acc.y), pack_bf16x2(acc.z, acc.w));
+      else
+        *reinterpret_cast<float4 *>(static_cast<float *>(dst) + r * D + d) = acc;
     }
   } else {
     const size_t n = rows * D;
@@ -1049,7 +1069,7 @@ __global__ __launch_bounds__(256) void head_sum_kernel(const float *__restrict__
       const int d = (int)(i - r * D);
       float acc = 0;
       for (int m = 0; m < M; ++m) acc += src[(r * M + m) * D + d];
-      dst[i] = acc;
+      static_cast<float *>(dst)[i] = acc;
     }
   }
 }
@@ -1141,6 +1161,7 @@ static size_t workspace_bytes_for(const BwdArgs &a, int kind, int dtype) {
   if (dtype == DFA3D_F64) return 0;
   if ((size_t)a.B * a.Q * a.M * a.L * a.P >= (1ull << 31)) return 0;          // point indices and segment offsets are 32-bit
   if (kind != 2 && (size_t)a.Q * a.M * a.C * 4 >= (size_t)kMaxSliceBytes) return 0;   // grad_out rows are buffer-addressed per batch element
+  if (a.grad_bf16 && (kind != 0 || ((a.C | a.D) & 3) != 0)) return 0;          // bfloat16 gradients: whole 8-byte groups
   const TileConfig c = tile_config_of(a, kind);
   if (c.lds > 150 * 1024) return 0;                                            // rows too long for LDS tiles
   return bin_layout(a, c.ty, c.tx).total;
@@ -1201,19 +1222,19 @@ static hipError_t launch_tile_cfg(const BwdArgs &a, const BinWorkspace &ws, cons
     auto kern = tile_backward_kernel<T, VEC, LPR, true>;
     if (hipError_t e = allow_lds(kern, c.lds)) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(c.block), c.lds, stream, ws, (const T *)a.value, (const T *)a.dist,
-                       (const T *)nullptr, (const T *)a.grad_out, (const T *)a.grad_score_in, (float *)a.grad_value,
-                       gd_heads != nullptr ? gd_heads : (float *)a.grad_dist, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
+                       (const T *)nullptr, (const T *)a.grad_out, (const T *)a.grad_score_in, a.grad_value,
+                       gd_heads != nullptr ? (void *)gd_heads : a.grad_dist, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
                        (float *)nullptr, (const float *)a.grad_weight_update, a.dist_heads == 1 ? 1 : a.M,
                        (a.dist_heads == 1 && gd_heads == nullptr) ? 1 : a.M, a.B, a.S, a.M, a.C, a.D, a.L, a.Q, a.P, c.pp,
-                       a.diag);
+                       (a.grad_bf16 ? 1 : 0) | ((a.grad_bf16 && gd_heads == nullptr) ? 2 : 0), a.diag);
   } else {
     auto kern = tile_backward_kernel<T, VEC, LPR, false>;
     if (hipError_t e = allow_lds(kern, c.lds)) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(c.block), c.lds, stream, ws, (const T *)a.value, (const T *)nullptr,
-                       (const T *)a.score_in, (const T *)a.grad_out, (const T *)nullptr, (float *)a.grad_value,
-                       (float *)nullptr, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
+                       (const T *)a.score_in, (const T *)a.grad_out, (const T *)nullptr, a.grad_value,
+                       (void *)nullptr, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
                        (float *)a.grad_score_out, (const float *)nullptr, a.M, a.M, a.B, a.S, a.M, a.C, 0, a.L, a.Q,
-                       a.P, c.pp, a.diag);
+                       a.P, c.pp, 0, a.diag);
   }
   return hipGetLastError();
 }
@@ -1296,11 +1317,12 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
   if (gd_heads != nullptr)       // a kernel, not a memset node: callers may capture this stream in a graph
     hipLaunchKernelGGL(fill_zero_kernel, dim3(2048), dim3(256), 0, stream, reinterpret_cast<float4 *>(gd_heads),
                        (head_floats + 3) / 4);
+  if (a.grad_bf16 && dtype != DFA3D_BF16) return hipErrorInvalidValue;
   const hipError_t e = dtype == DFA3D_F32 ? launch_tile_typed<float>(a, ws, cfg, gd_heads, stream)
                                           : launch_tile_typed<__hip_bfloat16>(a, ws, cfg, gd_heads, stream);
   if (e != hipSuccess || gd_heads == nullptr) return e;
-  hipLaunchKernelGGL(head_sum_kernel, dim3(2048), dim3(256), 0, stream, gd_heads, (float *)a.grad_dist,
-                     (size_t)a.B * a.S, a.M, a.D);
+  hipLaunchKernelGGL(head_sum_kernel, dim3(2048), dim3(256), 0, stream, gd_heads, a.grad_dist,
+                     (size_t)a.B * a.S, a.M, a.D, a.grad_bf16 ? 1 : 0);
   return hipGetLastError();
 }
 

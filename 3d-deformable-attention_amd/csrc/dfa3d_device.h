@@ -206,6 +206,20 @@ __device__ __forceinline__ void scatter_add(rsrc_t, double *base, uint32_t off, 
   if (off < kNoChan) unsafeAtomicAdd(reinterpret_cast<double *>(reinterpret_cast<char *>(base) + off), v);
 }
 
+// bfloat16 gradient storage (DFA3D_BF16G): two values rounded to nearest even and packed, and the
+// hardware's packed bfloat16 add on device memory (each add rounds the stored sum to bfloat16 again).
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  bf16x2_t v;
+  v.x = (__bf16)a; v.y = (__bf16)b;
+  return __builtin_bit_cast(uint32_t, v);
+}
+__device__ __forceinline__ void atomic_add_bf16x2(void *p, float a, float b) {
+  bf16x2_t v;
+  v.x = (__bf16)a; v.y = (__bf16)b;
+  __builtin_amdgcn_global_atomic_fadd_v2bf16(reinterpret_cast<bf16x2_t *>(p), v);
+}
+
 // ---------------------------------------------------------------------------------------
 // wave-private LDS hand-over between phases: LDS operations of one wavefront execute in
 // program order, so only the compiler has to be kept from moving accesses across the point.

@@ -65,6 +65,7 @@ struct BwdArgs {
   void *grad_attn, *grad_score_out;
   const void *grad_weight_update;    // gradient arriving at the forward's weight_update output, or nullptr
   int dist_heads;                    // as in FwdArgs; grad_dist has the same head count
+  int grad_bf16;                     // grad_value / grad_dist are bfloat16 (binned fused backward on bfloat16 storage only)
   int B, S, M, C, D, L, Q, P;
   int iters;
   int vec_hint;

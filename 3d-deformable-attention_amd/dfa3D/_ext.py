@@ -21,7 +21,7 @@ from . import _lib
 __all__ = [
     "wms_deform_attn_forward", "wms_deform_attn_backward",
     "ms_depth_score_sample_forward", "ms_depth_score_sample_backward",
-    "dfa3d_fused_forward", "dfa3d_fused_backward",
+    "dfa3d_fused_forward", "dfa3d_fused_backward", "fused_backward_grad_dtype",
 ]
 
 
@@ -324,11 +324,26 @@ def dfa3d_fused_forward(value, value_dpt_dist, value_spatial_shapes, value_level
     return (out, score, wu) if need_weight_update else (out, score)
 
 
+def fused_backward_grad_dtype(value, value_dpt_dist, sampling_locations):
+    """dtype the one-kernel backward can write grad_value / grad_value_dpt_dist in for these operands: bfloat16 for
+    bfloat16 storage when the LDS-tile kernels apply (the gradients then need no conversion pass before autograd
+    hands them on), else the accumulation type (float32 / float64)."""
+    aux = _aux_dtype(value.dtype)
+    if value.dtype != torch.bfloat16 or sampling_locations.numel() == 0:
+        return aux
+    B, S, M, C = value.shape
+    _, Q, _, L, P, _ = sampling_locations.shape
+    n = _lib.lib().dfa3d_fused_backward_workspace_bytes(B, S, M, C, value_dpt_dist.shape[3], L, Q, P,
+                                                        value_dpt_dist.shape[2], _lib.DFA3D_BF16G, _lib.options())
+    return torch.bfloat16 if n > 0 else aux
+
+
 def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
                          attention_weights, grad_output, grad_depth_score, grad_value, grad_value_dpt_dist,
                          grad_sampling_loc, grad_attn_weight, im2col_step, grad_weight_update=None):
     """One-kernel DFA3D backward.  ``grad_depth_score`` and ``grad_weight_update`` (gradients arriving at the
-    depth_score and weight_update outputs) may be None.  Accumulates into ``grad_value`` / ``grad_value_dpt_dist`` (pre-zeroed by the caller);
+    depth_score and weight_update outputs) may be None.  Accumulates into ``grad_value`` / ``grad_value_dpt_dist``
+    (pre-zeroed by the caller; float32 / float64, or both bfloat16 where ``fused_backward_grad_dtype`` says so);
     overwrites ``grad_sampling_loc`` (…, 3) and ``grad_attn_weight``."""
     named = dict(value=value, value_dpt_dist=value_dpt_dist, spatial_shapes=value_spatial_shapes,
                  level_start_index=value_level_start_index, sampling_loc=sampling_locations,
@@ -353,14 +368,15 @@ def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_leve
         if grad_weight_update.numel() != B * Q * M:
             raise RuntimeError(f"grad_weight_update has {grad_weight_update.numel()} elements, expected {B * Q * M}")
         _expect(grad_weight_update, "grad_weight_update", dtype=aux)
-    _expect(grad_value, "grad_value", shape=value.shape, dtype=aux)
-    _expect(grad_value_dpt_dist, "grad_value_dpt_dist", shape=value_dpt_dist.shape, dtype=aux)
+    g16 = value.dtype == torch.bfloat16 and grad_value.dtype == torch.bfloat16
+    _expect(grad_value, "grad_value", shape=value.shape, dtype=torch.bfloat16 if g16 else aux)
+    _expect(grad_value_dpt_dist, "grad_value_dpt_dist", shape=value_dpt_dist.shape, dtype=torch.bfloat16 if g16 else aux)
     _expect(grad_sampling_loc, "grad_sampling_loc", shape=(B, Q, M, L, P, 3), dtype=aux)
     _expect(grad_attn_weight, "grad_attn_weight", shape=(B, Q, M, L, P), dtype=aux)
     _step(B, im2col_step)
     if grad_output.numel() == 0:
         return
-    code = _lib.dtype_code(value)
+    code = _lib.DFA3D_BF16G if g16 else _lib.dtype_code(value)
     # scratch for the binned (LDS-accumulating) kernels; 0 bytes means the direct kernel is used
     ws_bytes = _lib.lib().dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2], code,
                                                                 _lib.options())

@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdfa3d_hip.so")
 
-DFA3D_F32, DFA3D_F64, DFA3D_BF16 = 0, 1, 2
+DFA3D_F32, DFA3D_F64, DFA3D_BF16, DFA3D_BF16G = 0, 1, 2, 3
 ABI_VERSION = 7
 
 _P, _I = ctypes.c_void_p, ctypes.c_int

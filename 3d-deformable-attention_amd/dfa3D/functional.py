@@ -25,7 +25,8 @@ and their ``_fp32`` / ``_fp16`` twins.  Differences from the reference, all on p
 * the ``_fp16`` twins cast to float32 under autocast: the reference's kernels are only instantiated
   for float and double (wms_deform_attn_cuda.cu:267), so its float16 twins cannot run at all;
 * bfloat16 ``value`` / ``value_dpt_dist`` (with float32 locations and attention weights) are accepted:
-  outputs come back in bfloat16, gradients are accumulated in float32 and cast on return.
+  outputs come back in bfloat16; gradients are accumulated in float32 and, in the one-kernel backward, rounded to
+  bfloat16 as the tiles are written (elsewhere: float32 buffers, cast on return).
 """
 import torch
 from torch.autograd.function import Function, once_differentiable
@@ -168,8 +169,9 @@ class MultiScale3DDeformableAttnFunction(Function):
         if grad_output is None:
             grad_output = torch.zeros(value.shape[0], sampling_locations.shape[1], value.shape[2] * value.shape[3],
                                       dtype=value.dtype, device=value.device)
-        grad_value = torch.zeros(value.shape, dtype=aux, device=value.device)
-        grad_value_dpt_dist = torch.zeros(value_dpt_dist.shape, dtype=aux, device=value.device)
+        gdt = _ext.fused_backward_grad_dtype(value, value_dpt_dist, sampling_locations)
+        grad_value = torch.zeros(value.shape, dtype=gdt, device=value.device)
+        grad_value_dpt_dist = torch.zeros(value_dpt_dist.shape, dtype=gdt, device=value.device)
         grad_sampling_loc = torch.empty_like(sampling_locations)
         grad_attn_weight = torch.empty_like(attention_weights)
         _ext.dfa3d_fused_backward(
@@ -211,8 +213,9 @@ class MultiScale3DDeformableAttnWeightUpdateFunction(Function):
         if grad_output is None:
             grad_output = torch.zeros(value.shape[0], sampling_locations.shape[1], value.shape[2] * value.shape[3],
                                       dtype=value.dtype, device=value.device)
-        grad_value = torch.zeros(value.shape, dtype=aux, device=value.device)
-        grad_value_dpt_dist = torch.zeros(value_dpt_dist.shape, dtype=aux, device=value.device)
+        gdt = _ext.fused_backward_grad_dtype(value, value_dpt_dist, sampling_locations)
+        grad_value = torch.zeros(value.shape, dtype=gdt, device=value.device)
+        grad_value_dpt_dist = torch.zeros(value_dpt_dist.shape, dtype=gdt, device=value.device)
         grad_sampling_loc = torch.empty_like(sampling_locations)
         grad_attn_weight = torch.empty_like(attention_weights)
         _ext.dfa3d_fused_backward(

@@ -502,8 +502,8 @@ def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
     B, S, M, C = value.shape
     D = dist.shape[3]
     _, Q, _, L, P, _ = loc.shape
-    code = _lib.dtype_code(value)
-    gdt = torch.float32
+    gdt = _ext.fused_backward_grad_dtype(value, dist, loc)          # bf16 storage: the kernel writes bf16 gradients
+    code = _lib.DFA3D_BF16G if gdt == torch.bfloat16 else _lib.dtype_code(value)
     gv = torch.zeros(value.shape, dtype=gdt, device=dev)
     gd = torch.zeros(dist.shape, dtype=gdt, device=dev)
     gl = torch.empty_like(loc)

@@ -25,6 +25,12 @@
  *     DFA3D_F64   every floating tensor double
  *     DFA3D_BF16  value, dist, out, score are bfloat16; loc, attn and EVERY gradient
  *                 buffer are float (accumulation is float throughout)
+ *     DFA3D_BF16G dfa3d_fused_backward / dfa3d_fused_backward_static only: as DFA3D_BF16, and grad_value and
+ *                 grad_dist are bfloat16 as well (what an autograd caller has to return for bfloat16 inputs):
+ *                 sums are formed in float in LDS and rounded once when a tile is written; the rows that
+ *                 several tiles share are added with the hardware's packed bfloat16 atomic, which rounds the
+ *                 stored sum at each of the few adds.  Offered on the binned kernels only
+ *                 (dfa3d_fused_backward_workspace_bytes(..., DFA3D_BF16G, ...) > 0: C and D multiples of 4)
  *
  * The four *_forward / *_backward pairs replace the reference's four native entry
  * points one for one; the two dfa3d_fused_* calls run both stages in one kernel.
@@ -42,6 +48,7 @@ extern "C" {
 #define DFA3D_F32 0
 #define DFA3D_F64 1
 #define DFA3D_BF16 2
+#define DFA3D_BF16G 3
 
 #define DFA3D_MAX_LEVELS 16
 

@@ -72,6 +72,11 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     assert L.dfa3d_fused_backward_workspace_bytes(*dims, 1, 0, None) > \
         L.dfa3d_fused_backward_workspace_bytes(*dims, 8, 0, None) > 0
     assert L.dfa3d_fused_backward_workspace_bytes(*dims, 8, 1, None) == 0    # fp64: direct kernels
+    # bfloat16 gradient buffers (DFA3D_BF16G = 3): fused backward only, C and D multiples of 4
+    assert L.dfa3d_fused_backward_workspace_bytes(*dims, 8, 3, None) == L.dfa3d_fused_backward_workspace_bytes(*dims, 8, 2, None)
+    assert L.dfa3d_fused_backward_workspace_bytes(6, 30825, 8, 32, 63, 4, 10000, 8, 8, 3, None) == 0
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 3, None, null)
+    assert rc == -1 and b"DFA3D_BF16G" in L.dfa3d_last_error()
 
 
 def test_launch_options_are_per_call_and_checked():
