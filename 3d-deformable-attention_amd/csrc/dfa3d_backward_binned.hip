@@ -1107,54 +1107,57 @@ static size_t tile_lds_bytes(int kind, int ty, int tx, int C, int D, int pp) {
   return (size_t)tile_lds_layout(ty, tx, C, kind == 1 ? 0 : D, pp).total * 4;
 }
 
-// Defaults: 512 threads, and the largest points-per-pass and tile whose LDS block still lets two workgroups
-// share a CU.  The staged grad_out rows take pp * C floats, so long rows first shorten the pass (256 -> 128 -> 64
-// points) and only then shrink the tile below 4 x 4 pixels.
-static TileConfig pick_tile_config(int kind, int C, int D, int tile_hint, int block_hint, int pass_hint) {
+// Defaults: 512 threads; the tile and the points per pass (pp) follow from what fits in LDS.  Measured on rows of
+// 32 .. 256 channels and 64 .. 256 depth bins: two workgroups per CU (79 KB each) beat one; passes of 64 points
+// lose to passes of 128 or 256 on any tile; with pp >= 128 the larger tile wins (8x8 at pp 128 over 4x8 at pp 256
+// for 128 bins); tiles below 4x4 pixels are several times slower than one workgroup per CU on a 4x8 tile (256
+// channels: 11.9 ms against 3.2 ms).  Hence the order below.
+// `dense`: so many points per pixel that most tiles take several passes; long passes then matter more than a large
+// tile (dense BEV workload, 41 points per pixel and 128 bins: 4x8 at pp 256 7.0 ms, 8x8 at pp 128 8.9 ms).
+static TileConfig pick_tile_config(int kind, int C, int D, int tile_hint, int block_hint, int pass_hint, bool dense) {
   TileConfig c;
   c.block = kind == 2 ? 256 : (block_hint == 256 ? 256 : 512);
   const int pp_max = kind == 2 ? c.block : c.block / 2;      // the fused tile kernel wants two halves of pp threads
   auto clamp_pp = [&](int pp) { return pp > pp_max ? pp_max : pp; };
   const int cand[][2] = {{16, 16}, {8, 16}, {8, 8}, {4, 8}, {4, 4}, {2, 4}, {2, 2}, {1, 1}};
-  const size_t budget = kind == 2 ? 40 * 1024 : 79 * 1024;
+  const size_t two_per_cu = kind == 2 ? 40 * 1024 : 79 * 1024, one_per_cu = 150 * 1024;
   const int hy = tile_hint / 100, hx = tile_hint % 100;
   const bool tile_given = tile_hint > 0 && hy >= 1 && hx >= 1 && hy <= 64 && hx <= 64;
   const bool pass_given = pass_hint == 64 || pass_hint == 128 || pass_hint == 256;
-  c.ty = c.tx = 1;
-  c.pp = clamp_pp(pass_given ? pass_hint : 256);
-  if (tile_given) { c.ty = hy; c.tx = hx; }
-  if (tile_given && pass_given) {
-  } else if (tile_given) {
-    for (int pp : {256, 128, 64}) {
-      c.pp = clamp_pp(pp);
-      if (tile_lds_bytes(kind, c.ty, c.tx, C, D, c.pp) <= budget) break;
-    }
-  } else {
-    bool found = false;
-    // tiles of at least 4 x 4 pixels with the longest pass that fits; then smaller tiles with the shortest
-    for (int round = 0; round < 2 && !found; ++round) {
-      for (int pp : {256, 128, 64}) {
-        if (pass_given && pp != pass_hint) continue;
-        if (!pass_given && round == 1 && pp != 64) continue;
-        for (auto &t : cand) {
-          if ((round == 0) != (t[0] * t[1] >= 16)) continue;
-          if (tile_lds_bytes(kind, t[0], t[1], C, D, clamp_pp(pp)) <= budget) {
-            c.ty = t[0]; c.tx = t[1]; c.pp = clamp_pp(pp); found = true;
-            break;
-          }
+  auto fits = [&](int ty, int tx, int pp, size_t budget) { return tile_lds_bytes(kind, ty, tx, C, D, clamp_pp(pp)) <= budget; };
+  auto done = [&](int ty, int tx, int pp) {
+    c.ty = ty; c.tx = tx; c.pp = clamp_pp(pp);
+    c.lds = tile_lds_bytes(kind, c.ty, c.tx, C, D, c.pp);
+    return c;
+  };
+  const int pp_order[3] = {256, 128, 64};
+  for (size_t budget : {two_per_cu, one_per_cu}) {
+    // classes of pass lengths, each tried on every tile before the next: {256, 128}, {64}; dense: {256}, {128}, {64}
+    const int n_cls = dense ? 3 : 2;
+    for (int cls = 0; cls < n_cls; ++cls) {
+      const int *pps = dense ? pp_order + cls : (cls == 0 ? pp_order : pp_order + 2);
+      const int n_pps = dense ? 1 : (cls == 0 ? 2 : 1);
+      for (auto &t : cand) {
+        if (tile_given ? (t[0] != cand[0][0] || t[1] != cand[0][1]) : (t[0] * t[1] < 16)) continue;   // a given tile: one turn
+        const int ty = tile_given ? hy : t[0], tx = tile_given ? hx : t[1];
+        for (int i = 0; i < n_pps; ++i) {
+          if (pass_given && pps[i] != pass_hint) continue;
+          if (fits(ty, tx, pps[i], budget)) return done(ty, tx, pps[i]);
         }
-        if (found) break;
       }
     }
-    if (!found) { c.ty = c.tx = 1; c.pp = clamp_pp(pass_given ? pass_hint : 64); }
   }
-  c.lds = tile_lds_bytes(kind, c.ty, c.tx, C, D, c.pp);
-  return c;
+  // nothing of at least 4x4 pixels fits: whatever the caller fixed, else the largest small tile with short passes
+  if (tile_given) return done(hy, hx, pass_given ? pass_hint : 64);
+  for (auto &t : cand)
+    if (t[0] * t[1] < 16 && fits(t[0], t[1], pass_given ? pass_hint : 64, one_per_cu)) return done(t[0], t[1], pass_given ? pass_hint : 64);
+  return done(1, 1, pass_given ? pass_hint : 64);
 }
 
 static int bwd_kind(const BwdArgs &a) { return a.dist != nullptr ? 0 : 1; }
 static TileConfig tile_config_of(const BwdArgs &a, int kind) {
-  return pick_tile_config(kind, a.C, a.D, a.tile_hint, a.block_hint, a.pass_hint);
+  const double per_pixel = (double)a.Q * a.L * a.P / (a.S > 0 ? a.S : 1);      // sampling points per pixel of a (batch, head)
+  return pick_tile_config(kind, a.C, a.D, a.tile_hint, a.block_hint, a.pass_hint, per_pixel >= 16.0);
 }
 
 static size_t workspace_bytes_for(const BwdArgs &a, int kind, int dtype) {
