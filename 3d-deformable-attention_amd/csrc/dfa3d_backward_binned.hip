@@ -1107,19 +1107,18 @@ static size_t tile_lds_bytes(int kind, int ty, int tx, int C, int D, int pp) {
   return (size_t)tile_lds_layout(ty, tx, C, kind == 1 ? 0 : D, pp).total * 4;
 }
 
-// Defaults: 512 threads; the tile and the points per pass (pp) follow from what fits in LDS.  Measured on rows of
-// 32 .. 256 channels and 64 .. 256 depth bins: two workgroups per CU (79 KB each) beat one; passes of 64 points
-// lose to passes of 128 or 256 on any tile; with pp >= 128 the larger tile wins (8x8 at pp 128 over 4x8 at pp 256
-// for 128 bins); tiles below 4x4 pixels are several times slower than one workgroup per CU on a 4x8 tile (256
-// channels: 11.9 ms against 3.2 ms).  Hence the order below.
-// `dense`: so many points per pixel that most tiles take several passes; long passes then matter more than a large
-// tile (dense BEV workload, 41 points per pixel and 128 bins: 4x8 at pp 256 7.0 ms, 8x8 at pp 128 8.9 ms).
+// Defaults: 512 threads; the tile and the points per pass (pp) follow from what fits in LDS, in an order of
+// preference taken from measurements on rows of 32 .. 256 channels and 64 .. 256 depth bins:
+//   * two workgroups per CU (79 KB each) beat one, and one per CU on a 4x8 tile beats tiles under 4x4 pixels by
+//     far (256 channels: 3.2 ms against 11.9 ms);
+//   * tiles above 8x16 pixels lose (the rows phase needs several rounds); passes of 64 points lose to 128 and 256;
+//   * an 8x8 tile at pp 128 beats a 4x8 tile at pp 256 (128 bins: 0.68 against 0.74 ms for 2.56 M points) unless
+//     most tiles take several passes (`dense`: the dense BEV workload, 41 points per pixel, 7.0 against 8.9 ms).
 static TileConfig pick_tile_config(int kind, int C, int D, int tile_hint, int block_hint, int pass_hint, bool dense) {
   TileConfig c;
   c.block = kind == 2 ? 256 : (block_hint == 256 ? 256 : 512);
   const int pp_max = kind == 2 ? c.block : c.block / 2;      // the fused tile kernel wants two halves of pp threads
   auto clamp_pp = [&](int pp) { return pp > pp_max ? pp_max : pp; };
-  const int cand[][2] = {{16, 16}, {8, 16}, {8, 8}, {4, 8}, {4, 4}, {2, 4}, {2, 2}, {1, 1}};
   const size_t two_per_cu = kind == 2 ? 40 * 1024 : 79 * 1024, one_per_cu = 150 * 1024;
   const int hy = tile_hint / 100, hx = tile_hint % 100;
   const bool tile_given = tile_hint > 0 && hy >= 1 && hx >= 1 && hy <= 64 && hx <= 64;
@@ -1130,28 +1129,26 @@ static TileConfig pick_tile_config(int kind, int C, int D, int tile_hint, int bl
     c.lds = tile_lds_bytes(kind, c.ty, c.tx, C, D, c.pp);
     return c;
   };
-  const int pp_order[3] = {256, 128, 64};
+  struct Pref { int ty, tx, pp; };
+  static const Pref sparse_order[] = {{8, 16, 256}, {8, 8, 256}, {8, 8, 128}, {4, 8, 256}, {4, 8, 128}, {4, 4, 256},
+                                      {4, 4, 128}, {8, 8, 64}, {4, 8, 64}, {4, 4, 64}};
+  static const Pref dense_order[] = {{8, 16, 256}, {8, 8, 256}, {4, 8, 256}, {4, 4, 256}, {8, 8, 128}, {4, 8, 128},
+                                     {4, 4, 128}, {8, 8, 64}, {4, 8, 64}, {4, 4, 64}};
+  const Pref *order = dense ? dense_order : sparse_order;
   for (size_t budget : {two_per_cu, one_per_cu}) {
-    // classes of pass lengths, each tried on every tile before the next: {256, 128}, {64}; dense: {256}, {128}, {64}
-    const int n_cls = dense ? 3 : 2;
-    for (int cls = 0; cls < n_cls; ++cls) {
-      const int *pps = dense ? pp_order + cls : (cls == 0 ? pp_order : pp_order + 2);
-      const int n_pps = dense ? 1 : (cls == 0 ? 2 : 1);
-      for (auto &t : cand) {
-        if (tile_given ? (t[0] != cand[0][0] || t[1] != cand[0][1]) : (t[0] * t[1] < 16)) continue;   // a given tile: one turn
-        const int ty = tile_given ? hy : t[0], tx = tile_given ? hx : t[1];
-        for (int i = 0; i < n_pps; ++i) {
-          if (pass_given && pps[i] != pass_hint) continue;
-          if (fits(ty, tx, pps[i], budget)) return done(ty, tx, pps[i]);
-        }
-      }
+    for (int i = 0; i < 10; ++i) {
+      const int ty = tile_given ? hy : order[i].ty, tx = tile_given ? hx : order[i].tx;
+      const int pp = pass_given ? pass_hint : order[i].pp;
+      if (fits(ty, tx, pp, budget)) return done(ty, tx, pp);
     }
   }
   // nothing of at least 4x4 pixels fits: whatever the caller fixed, else the largest small tile with short passes
-  if (tile_given) return done(hy, hx, pass_given ? pass_hint : 64);
-  for (auto &t : cand)
-    if (t[0] * t[1] < 16 && fits(t[0], t[1], pass_given ? pass_hint : 64, one_per_cu)) return done(t[0], t[1], pass_given ? pass_hint : 64);
-  return done(1, 1, pass_given ? pass_hint : 64);
+  const int pp = pass_given ? pass_hint : 64;
+  if (tile_given) return done(hy, hx, pp);
+  const int small[][2] = {{2, 4}, {2, 2}, {1, 1}};
+  for (auto &t : small)
+    if (fits(t[0], t[1], pp, one_per_cu)) return done(t[0], t[1], pp);
+  return done(1, 1, pp);
 }
 
 static int bwd_kind(const BwdArgs &a) { return a.dist != nullptr ? 0 : 1; }

@@ -384,7 +384,7 @@ def event_time(fn, reps, prep=None):
 def cpu_baseline(w, budget_s):
     """Forward+backward of the C restatement on a bounded sample (fewer queries, same everything else)."""
     import torch
-    from dfa3D.workloads import make_inputs, scaled
+    from dfa3D.workloads import WORKLOADS, make_inputs, scaled
     from oracle import dfa3d_oracle as orc
     threads = max(1, min(os.cpu_count() or 1, 64))
     orc.set_threads(threads)
@@ -402,7 +402,18 @@ def cpu_baseline(w, budget_s):
         spent += time.perf_counter() - t0
         reps += 1
     per_step = spent / reps
+    # the CPU-sized configuration in full (forward, as the reference's own test would run it)
+    unit = make_inputs(WORKLOADS["unit"])
+    uargs = (unit["value"], unit["value_dpt_dist"], unit["spatial_shapes"], unit["level_start_index"],
+             unit["sampling_locations"], unit["attention_weights"])
+    orc.dfa3d_forward(*uargs)
+    t0 = time.perf_counter()
+    for _ in range(50):
+        orc.dfa3d_forward(*uargs)
+    unit_ms = (time.perf_counter() - t0) * 1e3 / 50
     return {"value": sample.points / per_step, "unit": "points/s", "cores": threads, "kind": "port",
+            "unit_workload_forward_ms": round(unit_ms, 4),
+            "unit_workload_forward_points_per_s": WORKLOADS["unit"].points / (unit_ms * 1e-3),
             "sample": f"{w.name} workload with Q={sample.Q} of {w.Q} queries per batch element "
                       f"({sample.points} points), forward+backward, {reps} repetition(s), {per_step * 1e3:.1f} ms each; "
                       f"OpenMP over units (forward) and over the {sample.B} batch elements (backward)"}
