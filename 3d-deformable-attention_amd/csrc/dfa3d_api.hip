@@ -97,7 +97,7 @@ int check_dims(const char *fn, int B, int S, int M, int width, int L, int Q, int
 extern "C" {
 
 const char *dfa3d_last_error(void) { return g_err; }
-int dfa3d_abi_version(void) { return 7; }
+int dfa3d_abi_version(void) { return 8; }
 
 #ifdef DFA3D_EXPERIMENT
 int dfa3d_experiment_set(const char *name, int value) {
@@ -223,8 +223,31 @@ int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int
   return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
 }
 
+// cells of a packed distribution: sum over levels of (H + 1)(W + 1) <= sum of (2 H W + 2) <= 2 S + 2 L
+static long long packed_cells_bound(int S, int L) { return 2LL * S + 2LL * L; }
+
+size_t dfa3d_packed_dist_bytes(int B, int S, int D, int L, int dtype) {
+  if (B <= 0 || S <= 0 || D < 2 || L <= 0 || L > DFA3D_MAX_LEVELS || (dtype != DFA3D_F32 && dtype != DFA3D_BF16)) return 0;
+  const long long slice = packed_cells_bound(S, L) * D * 4 * (dtype == DFA3D_F32 ? 4 : 2);
+  if (slice >= (1LL << 30)) return 0;
+  return (size_t)slice * B;
+}
+
+int dfa3d_pack_dist(const void *dist, const int64_t *shapes3, const int64_t *level_start, void *packed,
+                    size_t packed_bytes, int B, int S, int D, int L, int dtype, void *stream) {
+  const char *fn = "dfa3d_pack_dist";
+  REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start); REQUIRE_PTR(fn, packed);
+  const size_t need = dfa3d_packed_dist_bytes(B, S, D, L, dtype);
+  if (need == 0)
+    return fail(DFA3D_EINVAL, "%s: not offered for these dimensions (needs D >= 2, DFA3D_F32 or DFA3D_BF16, and a batch "
+                "element of the packed table below 2^30 bytes)", fn);
+  if (packed_bytes < need) return fail(DFA3D_EINVAL, "%s: packed holds %zu bytes, %zu are needed", fn, packed_bytes, need);
+  return hip_result(dfa3d::launch_pack_dist(dist, shapes3, level_start, packed, B, S, D, L, dtype, (hipStream_t)stream), fn);
+}
+
 int dfa3d_fused_forward(const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
-                        const void *loc3, const void *attn, void *out, void *score, void *weight_update, int B, int S,
+                        const void *loc3, const void *attn, void *out, void *score, void *weight_update,
+                        const void *packed_dist, int B, int S,
                         int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype,
                         const dfa3d_launch_options *opts, void *stream) {
   const char *fn = "dfa3d_fused_forward";
@@ -233,12 +256,14 @@ int dfa3d_fused_forward(const void *value, const void *dist, const int64_t *shap
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
   if (int rc = check_opts(fn, opts, &o)) return rc;
   if (dist_heads != M && dist_heads != 1) return fail(DFA3D_EINVAL, "%s: dist_heads must be M or 1", fn);
+  if (packed_dist != nullptr && (dist_heads != 1 || dfa3d_packed_dist_bytes(B, S, D, L, dtype) == 0))
+    return fail(DFA3D_EINVAL, "%s: packed_dist goes with dist_heads = 1 and dimensions dfa3d_packed_dist_bytes accepts", fn);
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
   REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, out);
   dfa3d::FwdArgs a{};
   a.value = value; a.dist = dist; a.shapes = shapes3; a.shape_stride = 3; a.level_start = level_start;
   a.loc = loc3; a.loc_stride = 3; a.attn = attn; a.score_in = nullptr; a.out = out; a.score_out = score;
-  a.weight_update = weight_update; a.dist_heads = dist_heads;
+  a.weight_update = weight_update; a.dist_heads = dist_heads; a.packed_dist = packed_dist;
   a.B = B; a.S = S; a.M = M; a.C = C; a.D = D; a.L = L; a.Q = Q; a.P = P;
   a.iters = o.iters; a.vec_hint = o.vec;
   return hip_result(dfa3d::launch_forward(a, dtype, (hipStream_t)stream), fn);

@@ -239,6 +239,7 @@ struct LevelTable {
   int W[DFA3D_MAX_LEVELS];
   int Dd[DFA3D_MAX_LEVELS];
   int start[DFA3D_MAX_LEVELS];
+  int cell[DFA3D_MAX_LEVELS + 1];   // packed distributions only (load_cell_starts): first cell of each level, total
 };
 
 __device__ __forceinline__ void load_level_table(LevelTable &tab, const int64_t *shapes, int shape_stride,
@@ -257,6 +258,47 @@ __device__ __forceinline__ void load_level_table(LevelTable &tab, const int64_t 
   }
   __syncthreads();
 }
+
+// A packed distribution (dfa3d_pack_dist) holds, for every base pixel (h0, w0) with -1 <= h0 < H and
+// -1 <= w0 < W of every level (a "cell") and every depth bin d, the distribution values of the four pixels
+// around it in slot order LT,RT,RB,LB (zero outside the map): 4 elements per (cell, bin), bins consecutive.
+// Cells are numbered level by level, (h0 + 1) * (W + 1) + (w0 + 1) within a level.
+__device__ __forceinline__ void load_cell_starts(LevelTable &tab, int L) {
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int l = 0; l < L; ++l) {
+      tab.cell[l] = acc;
+      acc += (tab.H[l] + 1) * (tab.W[l] + 1);
+    }
+    tab.cell[L] = acc;
+  }
+  __syncthreads();
+}
+
+// bins (d, d + 1) of one cell: 8 elements, 32 bytes (16 for bfloat16), one cache line access
+template <typename T> struct PackedTap;
+template <> struct PackedTap<float> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, float (&x)[4], float (&y)[4]) {
+    const u32x4 t0 = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    const u32x4 t1 = __builtin_amdgcn_raw_buffer_load_b128(r, off == kNoRow ? kNoRow : off + 16, 0, 0);
+    x[0] = __uint_as_float(t0.x); x[1] = __uint_as_float(t0.y); x[2] = __uint_as_float(t0.z); x[3] = __uint_as_float(t0.w);
+    y[0] = __uint_as_float(t1.x); y[1] = __uint_as_float(t1.y); y[2] = __uint_as_float(t1.z); y[3] = __uint_as_float(t1.w);
+  }
+};
+template <> struct PackedTap<__hip_bfloat16> {
+  static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, float (&x)[4], float (&y)[4]) {
+    const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    x[0] = __uint_as_float(t.x << 16); x[1] = __uint_as_float(t.x & 0xFFFF0000u);
+    x[2] = __uint_as_float(t.y << 16); x[3] = __uint_as_float(t.y & 0xFFFF0000u);
+    y[0] = __uint_as_float(t.z << 16); y[1] = __uint_as_float(t.z & 0xFFFF0000u);
+    y[2] = __uint_as_float(t.w << 16); y[3] = __uint_as_float(t.w & 0xFFFF0000u);
+  }
+};
+template <> struct PackedTap<double> {      // not offered (the launcher never passes a packed table of doubles)
+  static __device__ __forceinline__ void ld(rsrc_t, uint32_t, double (&x)[4], double (&y)[4]) {
+    for (int k = 0; k < 4; ++k) { x[k] = 0; y[k] = 0; }
+  }
+};
 
 // ---------------------------------------------------------------------------------------
 // geometry of one sampling point
@@ -376,6 +418,10 @@ template <> struct BufPair<__hip_bfloat16> {
   }
 };
 
+// score of a corner from its two taps, written so that every kernel rounds it the same way
+__device__ __forceinline__ float depth_lerp(float lo, float hi, float hd, float ld) { return __builtin_fmaf(hi, ld, lo * hd); }
+__device__ __forceinline__ double depth_lerp(double lo, double hi, double hd, double ld) { return __builtin_fma(hi, ld, lo * hd); }
+
 // LOCAL: the caller's taps mostly hit lines its workgroup has just used (tile kernels)
 template <typename T, bool LOCAL> struct PairLoader {
   static __device__ __forceinline__ void ld(rsrc_t r, uint32_t off, int, T &x, T &y) { BufPair<T>::ld(r, off, x, y); }
@@ -417,7 +463,7 @@ __device__ __forceinline__ void corner_scores(rsrc_t dist_r, const int (&key)[4]
     }
   }
 #pragma unroll
-  for (int k = 0; k < 4; ++k) score[k] = lo[k] * tap.hd + hi[k] * tap.ld;
+  for (int k = 0; k < 4; ++k) score[k] = depth_lerp(lo[k], hi[k], tap.hd, tap.ld);
 }
 
 // one task of phase B: byte offset of a value row inside the batch element (kNoRow = nothing

@@ -56,12 +56,14 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
     const T *__restrict__ value, const T *__restrict__ dist, const int64_t *__restrict__ shapes, int shape_stride,
     const int64_t *__restrict__ level_start, const A *__restrict__ loc, int loc_stride,
     const A *__restrict__ attn, const T *__restrict__ score_in, T *__restrict__ out, T *__restrict__ score_out,
-    A *__restrict__ weight_update, int Md, int B, int S, int M, int C, int D, int L, int Q, int P, int iters,
-    int q_blocks) {
+    A *__restrict__ weight_update, const T *__restrict__ packed, int Md, int B, int S, int M, int C, int D, int L,
+    int Q, int P, int iters, int q_blocks) {
+  // packed: the head-shared distribution as dfa3d_pack_dist lays it out (D >= 2), or nullptr
   __shared__ LevelTable tab;
   __shared__ Task<A> s_tasks[kWavesPerBlock][kWave * 4];
 
   load_level_table(tab, shapes, shape_stride, level_start, L, S, FUSED ? D : 0);
+  if (FUSED && packed != nullptr) load_cell_starts(tab, L);          // uniform
 
   const WaveShape ws = wave_shape(L, P);
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -76,6 +78,8 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
   const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * Md * D : nullptr,
                                   FUSED ? (size_t)S * Md * D * sizeof(T) : 0);
   const int md = Md == 1 ? 0 : m;                                    // head whose distribution this head reads
+  const size_t packed_slice = (FUSED && packed != nullptr) ? (size_t)tab.cell[L] * D * 4 : 0;   // elements per batch element
+  const rsrc_t packed_r = make_rsrc(packed_slice ? packed + (size_t)b * packed_slice : nullptr, packed_slice * sizeof(T));
   const int q_per_iter = kWavesPerBlock * ws.upw;
 
   for (int it = 0; it < iters; ++it) {
@@ -113,7 +117,23 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
           if (FUSED) {
             A lo[4], hi[4];
             const DepthTap<A> tap = locate_depth<A>(__builtin_nontemporal_load(pl + 2), tab.Dd[l]);
-            corner_scores<T, A>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
+            if (packed != nullptr) {                                // uniform: all eight taps from one line
+              const int db = min(max(tap.d0, 0), D - 2);
+              const bool lo_x = tap.lo_ok && tap.d0 == db, lo_y = tap.lo_ok && tap.d0 == db + 1;
+              const bool hi_x = tap.hi_ok && tap.d0 + 1 == db, hi_y = tap.hi_ok && tap.d0 + 1 == db + 1;
+              const int cell = tab.cell[l] + (g.h0 + 1) * (tab.W[l] + 1) + g.w0 + 1;
+              A x4[4], y4[4];
+              PackedTap<T>::ld(packed_r, (g.inside && tap.inside) ? (uint32_t)((cell * D + db) * 4 * (int)sizeof(T)) : kNoRow,
+                               x4, y4);
+#pragma unroll
+              for (int k = 0; k < 4; ++k) {
+                lo[k] = lo_x ? x4[k] : lo_y ? y4[k] : (A)0;
+                hi[k] = hi_x ? x4[k] : hi_y ? y4[k] : (A)0;
+                sc[k] = depth_lerp(lo[k], hi[k], tap.hd, tap.ld);
+              }
+            } else {
+              corner_scores<T, A>(dist_r, g.key, tap, md, Md, D, sc, lo, hi);
+            }
             if (score_out != nullptr && pass == 0) {
               T *so = score_out + gp * 4;
               if constexpr (sizeof(T) == 4) {                     // one 16-byte store
@@ -232,6 +252,59 @@ __global__ __launch_bounds__(kBlock) void depth_score_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
+// Packs a head-shared distribution (B,S,1,D) for the forward's depth taps: see load_cell_starts for the layout.
+// One thread per (cell, bin): four gathered values, one 16-byte (bfloat16: 8-byte) store; consecutive threads
+// write consecutive addresses.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void pack_dist_kernel(
+    const T *__restrict__ dist, const int64_t *__restrict__ shapes3, const int64_t *__restrict__ level_start,
+    T *__restrict__ packed, int B, int S, int D, int L) {
+  __shared__ LevelTable tab;
+  load_level_table(tab, shapes3, 3, level_start, L, S, D);
+  load_cell_starts(tab, L);
+  const size_t cells = (size_t)tab.cell[L];
+  const size_t n = (size_t)B * cells * D;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const int d = (int)(i % D);
+    const size_t bc = i / D;
+    const int cell = (int)(bc % cells), b = (int)(bc / cells);
+    int l = 0;
+    while (l + 1 < L && cell >= tab.cell[l + 1]) ++l;
+    const int H = tab.H[l], W = tab.W[l], local = cell - tab.cell[l];
+    const int h0 = local / (W + 1) - 1, w0 = local % (W + 1) - 1;
+    const T *lvl = dist + ((size_t)b * S + tab.start[l]) * D + d;
+    T v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int h = h0 + (k >= 2 ? 1 : 0), w = w0 + ((k == 1 || k == 2) ? 1 : 0);      // slots LT, RT, RB, LB
+      const bool in = h >= 0 && h < H && w >= 0 && w < W;
+      v[k] = in ? lvl[(size_t)(h * W + w) * D] : T(0.f);
+    }
+    T *dst = packed + i * 4;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) dst[k] = v[k];
+  }
+}
+
+template <typename T>
+static hipError_t launch_pack_typed(const void *dist, const int64_t *shapes3, const int64_t *level_start, void *packed,
+                                    int B, int S, int D, int L, hipStream_t stream) {
+  hipLaunchKernelGGL((pack_dist_kernel<T>), dim3(256 * 16), dim3(256), 0, stream, (const T *)dist, shapes3, level_start,
+                     (T *)packed, B, S, D, L);
+  return hipGetLastError();
+}
+
+hipError_t launch_pack_dist(const void *dist, const int64_t *shapes3, const int64_t *level_start, void *packed, int B,
+                            int S, int D, int L, int dtype, hipStream_t stream) {
+  switch (dtype) {
+    case DFA3D_F32: return launch_pack_typed<float>(dist, shapes3, level_start, packed, B, S, D, L, stream);
+    case DFA3D_BF16: return launch_pack_typed<__hip_bfloat16>(dist, shapes3, level_start, packed, B, S, D, L, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+// ---------------------------------------------------------------------------------------
 // launchers
 // ---------------------------------------------------------------------------------------
 template <typename T, typename A, int VEC, int LPR>
@@ -246,13 +319,14 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
     hipLaunchKernelGGL((fwd_attention_kernel<T, A, VEC, LPR, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,
                        (const T *)a.value, (const T *)a.dist, a.shapes, a.shape_stride, a.level_start,
                        (const A *)a.loc, a.loc_stride, (const A *)a.attn, (const T *)nullptr, (T *)a.out,
-                       (T *)a.score_out, (A *)a.weight_update, a.dist_heads == 1 ? 1 : a.M, a.B, a.S, a.M, a.C, a.D,
-                       a.L, a.Q, a.P, iters, q_blocks);
+                       (T *)a.score_out, (A *)a.weight_update, (const T *)a.packed_dist, a.dist_heads == 1 ? 1 : a.M, a.B,
+                       a.S, a.M, a.C, a.D, a.L, a.Q, a.P, iters, q_blocks);
   } else {
     hipLaunchKernelGGL((fwd_attention_kernel<T, A, VEC, LPR, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,
                        (const T *)a.value, (const T *)nullptr, a.shapes, a.shape_stride, a.level_start,
                        (const A *)a.loc, a.loc_stride, (const A *)a.attn, (const T *)a.score_in, (T *)a.out,
-                       (T *)nullptr, (A *)nullptr, a.M, a.B, a.S, a.M, a.C, a.D, a.L, a.Q, a.P, iters, q_blocks);
+                       (T *)nullptr, (A *)nullptr, (const T *)nullptr, a.M, a.B, a.S, a.M, a.C, a.D, a.L, a.Q, a.P, iters,
+                       q_blocks);
   }
   return hipGetLastError();
 }

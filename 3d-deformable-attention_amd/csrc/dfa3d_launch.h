@@ -44,6 +44,7 @@ struct FwdArgs {
   void *out, *score_out;             // score_out may be nullptr
   void *weight_update;               // (B,Q,M) sum over a unit's points of attn * mean corner score, or nullptr
   int dist_heads;                    // heads stored in dist: M, or 1 for one distribution shared by all heads
+  const void *packed_dist;           // dist_heads == 1 only: the distribution as dfa3d_pack_dist lays it out, or nullptr
   int B, S, M, C, D, L, Q, P;
   int iters;                         // groups of units each wavefront walks through
   int vec_hint;
@@ -85,6 +86,8 @@ struct DepthScoreBwdArgs {
 };
 
 hipError_t launch_forward(const FwdArgs &a, int dtype, hipStream_t stream);
+hipError_t launch_pack_dist(const void *dist, const int64_t *shapes3, const int64_t *level_start, void *packed, int B,
+                            int S, int D, int L, int dtype, hipStream_t stream);
 hipError_t launch_depth_score(const DepthScoreArgs &a, int dtype, hipStream_t stream);
 hipError_t launch_backward(const BwdArgs &a, int dtype, hipStream_t stream);
 hipError_t launch_depth_score_backward(const DepthScoreBwdArgs &a, int dtype, hipStream_t stream);

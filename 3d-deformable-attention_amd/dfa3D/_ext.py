@@ -21,7 +21,7 @@ from . import _lib
 __all__ = [
     "wms_deform_attn_forward", "wms_deform_attn_backward",
     "ms_depth_score_sample_forward", "ms_depth_score_sample_backward",
-    "dfa3d_fused_forward", "dfa3d_fused_backward", "fused_backward_grad_dtype",
+    "dfa3d_fused_forward", "dfa3d_fused_backward", "fused_backward_grad_dtype", "pack_shared_dist",
 ]
 
 
@@ -295,12 +295,41 @@ def _fused_dims(value, dist, shapes3, lsi, loc3, attn, name):
     return B, S, M, C, D, L, Q, P
 
 
+def pack_shared_dist(value_dpt_dist, value_spatial_shapes, value_level_start_index):
+    """A distribution shared by all heads, (bs, keys, 1, D), laid out for the forward's depth taps (the four pixels
+    around every base pixel side by side, per bin): pass the result as ``packed_dist`` to ``dfa3d_fused_forward``.
+    Returns None where the library does not offer it (D < 2, float64).  Worth keeping: every forward on the same
+    distribution (DFA3D-BEVFormer runs six encoder layers on one) can use the same packed tensor."""
+    _contig(value_dpt_dist=value_dpt_dist, spatial_shapes=value_spatial_shapes,
+            level_start_index=value_level_start_index)
+    dev = _on_gpu(value_dpt_dist=value_dpt_dist, spatial_shapes=value_spatial_shapes,
+                  level_start_index=value_level_start_index)
+    if value_dpt_dist.dim() != 4 or value_dpt_dist.shape[2] != 1:
+        raise RuntimeError(f"value_dpt_dist must be (bs, keys, 1, D), got {tuple(value_dpt_dist.shape)}")
+    if value_dpt_dist.dtype == torch.float64:
+        return None
+    B, S, _, D = value_dpt_dist.shape
+    L = value_spatial_shapes.shape[0]
+    code = _lib.dtype_code(value_dpt_dist)
+    n = _lib.lib().dfa3d_packed_dist_bytes(B, S, D, L, code)
+    if n == 0:
+        return None
+    packed = torch.empty(n, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().dfa3d_pack_dist(_lib.ptr(value_dpt_dist), _lib.ptr(value_spatial_shapes),
+                                        _lib.ptr(value_level_start_index), _lib.ptr(packed), n, B, S, D, L, code,
+                                        _lib.stream_of(value_dpt_dist))
+    _lib.check(rc, "dfa3d_pack_dist")
+    return packed
+
+
 def dfa3d_fused_forward(value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
-                        attention_weights, im2col_step, need_depth_score=True, need_weight_update=False):
+                        attention_weights, im2col_step, need_depth_score=True, need_weight_update=False,
+                        packed_dist=None):
     """One-kernel DFA3D forward -> (output (bs, Q, heads*C), depth_score (bs, Q, heads, L, P, 4) or None), and
     with ``need_weight_update`` a third result, weight_update (bs, Q, heads, 1) = sum over levels and points of
     attention weight * mean corner score.  ``value_dpt_dist`` is (bs, keys, heads, D), or (bs, keys, 1, D) for one
-    distribution shared by all heads."""
+    distribution shared by all heads; for the latter ``packed_dist`` may be what ``pack_shared_dist`` returned for it."""
     _contig(value=value, value_dpt_dist=value_dpt_dist, spatial_shapes=value_spatial_shapes,
             level_start_index=value_level_start_index, sampling_loc=sampling_locations, attn_weight=attention_weights)
     dev = _on_gpu(value=value, value_dpt_dist=value_dpt_dist, spatial_shapes=value_spatial_shapes,
@@ -309,6 +338,13 @@ def dfa3d_fused_forward(value, value_dpt_dist, value_spatial_shapes, value_level
     B, S, M, C, D, L, Q, P = _fused_dims(value, value_dpt_dist, value_spatial_shapes, value_level_start_index,
                                          sampling_locations, attention_weights, "dfa3d_fused_forward")
     _step(B, im2col_step)
+    if packed_dist is not None:
+        if value_dpt_dist.shape[2] != 1:
+            raise RuntimeError("packed_dist goes with a distribution shared by all heads, (bs, keys, 1, D)")
+        need = _lib.lib().dfa3d_packed_dist_bytes(B, S, D, L, _lib.dtype_code(value))
+        if need == 0 or packed_dist.device != dev or not packed_dist.is_contiguous() or \
+                packed_dist.numel() * packed_dist.element_size() < need:
+            raise RuntimeError(f"packed_dist must be a contiguous tensor of at least {need} bytes on {dev}")
     out = torch.empty(B, Q, M * C, dtype=value.dtype, device=dev)
     score = torch.empty(B, Q, M, L, P, 4, dtype=value.dtype, device=dev) if need_depth_score else None
     wu = torch.empty(B, Q, M, 1, dtype=_aux_dtype(value.dtype), device=dev) if need_weight_update else None
@@ -318,7 +354,8 @@ def dfa3d_fused_forward(value, value_dpt_dist, value_spatial_shapes, value_level
         rc = _lib.lib().dfa3d_fused_forward(
             _lib.ptr(value), _lib.ptr(value_dpt_dist), _lib.ptr(value_spatial_shapes),
             _lib.ptr(value_level_start_index), _lib.ptr(sampling_locations), _lib.ptr(attention_weights),
-            _lib.ptr(out), _lib.ptr(score), _lib.ptr(wu), B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2],
+            _lib.ptr(out), _lib.ptr(score), _lib.ptr(wu), _lib.ptr(packed_dist), B, S, M, C, D, L, Q, P,
+            value_dpt_dist.shape[2],
             _lib.dtype_code(value), _lib.options(), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_fused_forward")
     return (out, score, wu) if need_weight_update else (out, score)

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdfa3d_hip.so")
 
 DFA3D_F32, DFA3D_F64, DFA3D_BF16, DFA3D_BF16G = 0, 1, 2, 3
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _P, _I = ctypes.c_void_p, ctypes.c_int
 _DIMS7 = [_I] * 7      # B S M (C|D) L Q P
@@ -36,7 +36,8 @@ SIGNATURES = {
     "dfa3d_wms_deform_attn_forward": [_P, _P, _I, _P, _P, _I, _P, _P, _P] + _DIMS7 + [_I, _O, _P],
     "dfa3d_wms_deform_attn_backward": [_P, _P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _P, ctypes.c_size_t]
     + _DIMS7 + [_I, _O, _P],
-    "dfa3d_fused_forward": [_P] * 9 + _DIMS8 + [_I, _I, _O, _P],
+    "dfa3d_fused_forward": [_P] * 10 + _DIMS8 + [_I, _I, _O, _P],
+    "dfa3d_pack_dist": [_P, _P, _P, _P, ctypes.c_size_t, _I, _I, _I, _I, _I, _P],
     "dfa3d_fused_backward": [_P] * 14 + [ctypes.c_size_t] + _DIMS8 + [_I, _I, _O, _P],
     "dfa3d_fused_backward_static": [_P] * 13 + _DIMS8 + [_I, _I, _O, _P],
     "dfa3d_rebatch_gather": [_P, ctypes.c_longlong, ctypes.c_longlong, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
@@ -66,6 +67,8 @@ def lib():
             fn = getattr(handle, name)
             fn.argtypes = dims + [_I, _O]
             fn.restype = ctypes.c_size_t
+        handle.dfa3d_packed_dist_bytes.argtypes = [_I] * 5
+        handle.dfa3d_packed_dist_bytes.restype = ctypes.c_size_t
         handle.dfa3d_static_scratch_bytes.argtypes = []
         handle.dfa3d_static_scratch_bytes.restype = ctypes.c_size_t
         handle.dfa3d_last_error.argtypes = []

@@ -49,6 +49,17 @@ def _aux(t):
     return torch.float32 if t.dtype == torch.bfloat16 else t.dtype
 
 
+def _packed_for_forward(value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations):
+    """The packed form of a distribution shared by all heads when making it pays for this call (its cost grows
+    with keys x bins, what it saves with the number of sampling points), else None."""
+    if value_dpt_dist.dim() != 4 or value_dpt_dist.shape[2] != 1 or not value_dpt_dist.is_cuda:
+        return None
+    B, S, _, D = value_dpt_dist.shape
+    if sampling_locations.numel() // 3 < B * S * D:
+        return None
+    return _ext.pack_shared_dist(value_dpt_dist, value_spatial_shapes, value_level_start_index)
+
+
 def _grad_in(g, like):
     """Incoming gradient as a contiguous tensor of the dtype the forward output had."""
     g = g.contiguous()
@@ -155,7 +166,9 @@ class MultiScale3DDeformableAttnFunction(Function):
         ctx.set_materialize_grads(False)
         output, depth_score = _ext.dfa3d_fused_forward(
             value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
-            attention_weights, im2col_step=ctx.im2col_step)
+            attention_weights, im2col_step=ctx.im2col_step,
+            packed_dist=_packed_for_forward(value_dpt_dist, value_spatial_shapes, value_level_start_index,
+                                            sampling_locations))
         ctx.save_for_backward(value, value_dpt_dist, value_spatial_shapes, value_level_start_index,
                               sampling_locations, attention_weights)
         return output, depth_score
@@ -190,16 +203,23 @@ class MultiScale3DDeformableAttnWeightUpdateFunction(Function):
     (BEVFormer_DFA3D/projects/mmdet3d_plugin/bevformer/modules/spatial_cross_attention.py:579), computed in the
     kernel so that the (bs, Q, heads, L, P, 4) score tensor is never written.  ``value_dpt_dist`` may be
     (bs, keys, 1, D): one distribution for all heads, without the repeat of spatial_cross_attention.py:496-497.
-    Both outputs are differentiable."""
+    Both outputs are differentiable.  An optional eighth argument is that distribution as
+    ``dfa3D._ext.pack_shared_dist`` lays it out for the forward's depth taps: a caller that runs several layers on
+    one distribution (DFA3D-BEVFormer's six encoder layers) packs once and passes it to each; without it the
+    forward packs for itself when that pays."""
 
     @staticmethod
     def forward(ctx, value, value_dpt_dist, value_spatial_shapes, value_level_start_index,
-                sampling_locations, attention_weights, im2col_step):
+                sampling_locations, attention_weights, im2col_step, packed_dist=None):
         ctx.im2col_step = im2col_step
         ctx.set_materialize_grads(False)
+        if packed_dist is None:
+            packed_dist = _packed_for_forward(value_dpt_dist, value_spatial_shapes, value_level_start_index,
+                                              sampling_locations)
         output, _, weight_update = _ext.dfa3d_fused_forward(
             value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
-            attention_weights, im2col_step=ctx.im2col_step, need_depth_score=False, need_weight_update=True)
+            attention_weights, im2col_step=ctx.im2col_step, need_depth_score=False, need_weight_update=True,
+            packed_dist=packed_dist)
         ctx.save_for_backward(value, value_dpt_dist, value_spatial_shapes, value_level_start_index,
                               sampling_locations, attention_weights)
         return output, weight_update.to(attention_weights.dtype)
@@ -223,8 +243,9 @@ class MultiScale3DDeformableAttnWeightUpdateFunction(Function):
             attention_weights, _grad_in(grad_output, value.dtype), None,
             grad_value, grad_value_dpt_dist, grad_sampling_loc, grad_attn_weight, im2col_step=ctx.im2col_step,
             grad_weight_update=None if grad_weight_update is None else _grad_in(grad_weight_update, aux))
-        return grad_value.to(value.dtype), grad_value_dpt_dist.to(value_dpt_dist.dtype), None, None, \
-            grad_sampling_loc, grad_attn_weight, None
+        # one gradient per forward argument: seven, or eight when the packed distribution was passed in
+        return (grad_value.to(value.dtype), grad_value_dpt_dist.to(value_dpt_dist.dtype), None, None,
+                grad_sampling_loc, grad_attn_weight, None, None)
 
 
 def _autocast_twin(base, name, doc):

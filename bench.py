@@ -333,6 +333,13 @@ def variant_timings(_ext, torch, value, dist, shapes, lsi, loc, attn, go, reps):
 
     out["shared_dist_weight_update_fwd_ms"] = round(event_time(lambda: _ext.dfa3d_fused_forward(
         value, shared, shapes, lsi, loc, attn, 64, need_depth_score=False, need_weight_update=True), reps)[0], 4)
+    packed = _ext.pack_shared_dist(shared, shapes, lsi)
+    if packed is not None:     # the same forward with its depth taps from the packed distribution, and the packing itself
+        out["shared_dist_packed_fwd_ms"] = round(event_time(lambda: _ext.dfa3d_fused_forward(
+            value, shared, shapes, lsi, loc, attn, 64, need_depth_score=False, need_weight_update=True,
+            packed_dist=packed), reps)[0], 4)
+        out["pack_shared_dist_ms"] = round(event_time(lambda: _ext.pack_shared_dist(shared, shapes, lsi), reps)[0], 4)
+    del packed
     out["shared_dist_bwd_ms"] = round(event_time(shared_bwd, reps)[0], 4)
 
     def plain_bwd():

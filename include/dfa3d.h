@@ -133,13 +133,29 @@ size_t dfa3d_wms_deform_attn_backward_workspace_bytes(int B, int S, int M, int C
  * all heads, dist (B,S,1,D): what the reference's caller builds with an 8-fold repeat
  * (BEVFormer_DFA3D/projects/mmdet3d_plugin/bevformer/modules/spatial_cross_attention.py:496-497).
  * weight_update[b,q,m] = sum over (l,p) of attn * mean of the four corner scores: the reduction that
- * caller applies to the score tensor right after the call (spatial_cross_attention.py:579). */
+ * caller applies to the score tensor right after the call (spatial_cross_attention.py:579).
+ *
+ * `packed_dist` (may be NULL; dist_heads = 1 only) is the same distribution as dfa3d_pack_dist lays it out: the
+ * eight depth taps of a sampling point then come from one cache line instead of four, and the distribution no
+ * longer competes with the value rows for the L2.  Results are identical. */
 int dfa3d_fused_forward(
     const void *value, const void *dist, const int64_t *shapes3, const int64_t *level_start,
     const void *loc3, const void *attn,
-    void *out, void *score, void *weight_update,
+    void *out, void *score, void *weight_update, const void *packed_dist,
     int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads, int dtype,
     const dfa3d_launch_options *opts, void *stream);
+
+/* Packs a distribution shared by all heads, dist (B,S,1,D), for the forward: for every level, every base pixel
+ * (h0, w0) with -1 <= h0 < H, -1 <= w0 < W and every bin d, the values of the four pixels (h0, w0), (h0, w0+1),
+ * (h0+1, w0+1), (h0+1, w0) side by side (zero outside the map), i.e. 4 (H+1)(W+1) D elements per level and batch
+ * element.  No counterpart in the reference, whose caller repeats the distribution per head instead
+ * (spatial_cross_attention.py:496-497).  A caller that runs several attention layers on one distribution
+ * (DFA3D-BEVFormer's six encoder layers do) packs once.  `packed` holds at least dfa3d_packed_dist_bytes(...)
+ * bytes (an upper bound from S and L, since the level shapes live on the device; 0 = not offered: D < 2,
+ * DFA3D_F64, or a batch element of the table at or above 2^30 bytes); every byte the forward reads is written. */
+size_t dfa3d_packed_dist_bytes(int B, int S, int D, int L, int dtype);
+int dfa3d_pack_dist(const void *dist, const int64_t *shapes3, const int64_t *level_start, void *packed,
+                    size_t packed_bytes, int B, int S, int D, int L, int dtype, void *stream);
 
 /* Backward of dfa3d_fused_forward (…_function.py:306-352: two native calls, six zero fills and
  * a host synchronisation in the reference).  The depth scores are recomputed from `dist`, not

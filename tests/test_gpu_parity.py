@@ -945,3 +945,66 @@ def test_bf16_gradients_in_float_buffers_and_in_bf16_buffers_agree(oracle):
     with pytest.raises(RuntimeError, match="DFA3D_BF16G"):
         _ext.dfa3d_fused_backward(v, d_odd, sh_odd, lsi, loc, at, go, None, gv, gd, torch.empty_like(loc),
                                   torch.empty_like(at), 64)
+
+
+@pytest.mark.parametrize("case", [dict(seed=201, B=2, M=4, C=8, D=2, Q=50, P=3, levels=((5, 7), (1, 1), (3, 2))),
+                                  dict(seed=202, B=1, M=8, C=32, D=64, Q=400, P=8, levels=((23, 31), (12, 16), (6, 8), (3, 4))),
+                                  dict(seed=203, B=3, M=3, C=16, D=17, Q=90, P=5, levels=((9, 4),), lo=-0.6, hi=1.6)],
+                         ids=lambda c: f"seed{c['seed']}")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_packed_shared_distribution_gives_identical_results(oracle, case, dtype):
+    """The forward with the distribution packed for its depth taps (dfa3d_pack_dist: one cache line per point
+    instead of four) against the forward that gathers from the distribution itself: bit-identical output, scores
+    and weight_update, out-of-range locations and one-pixel levels included; and against the checker."""
+    from dfa3D import _ext
+    dev = _dev()
+    t = tiny_case(dtype=torch.float32, **case)
+    inp = _as_inputs(t)
+    v, d = inp["value"].to(dtype).to(dev), inp["value_dpt_dist"][:, :, :1].contiguous().to(dtype).to(dev)
+    sh, lsi = inp["spatial_shapes"].to(dev), inp["level_start_index"].to(dev)
+    loc, at = inp["sampling_locations"].to(dev), inp["attention_weights"].to(dev)
+    packed = _ext.pack_shared_dist(d, sh, lsi)
+    assert packed is not None
+    plain = _ext.dfa3d_fused_forward(v, d, sh, lsi, loc, at, 64, need_weight_update=True)
+    fast = _ext.dfa3d_fused_forward(v, d, sh, lsi, loc, at, 64, need_weight_update=True, packed_dist=packed)
+    for a, b, name in zip(plain, fast, ("output", "depth_score", "weight_update")):
+        assert torch.equal(a, b), name
+    if dtype == torch.float32:
+        shared = dict(inp, value_dpt_dist=inp["value_dpt_dist"][:, :, :1].contiguous())
+        want = _shared_dist_expectation(oracle, shared)
+        torch.testing.assert_close(fast[0].cpu(), want[0], **F32_FWD)
+        torch.testing.assert_close(fast[1].cpu(), want[1], **F32_FWD)
+        torch.testing.assert_close(fast[2].cpu(), want[2], **F32_FWD)
+
+
+def test_packed_distribution_through_the_functions_and_refusals():
+    """The weight_update Function takes the packed distribution as an optional eighth argument (one packing for
+    several layers) and packs for itself otherwise; both give the gradients of the call without packing.  A single
+    depth bin and float64 are not offered; a packed table with a distribution per head is refused."""
+    from dfa3D import _ext
+    from dfa3D.functional import MultiScale3DDeformableAttnWeightUpdateFunction as F
+    from dfa3D.workloads import WORKLOADS, make_inputs, scaled
+    dev = _dev()
+    inp = make_inputs(scaled(WORKLOADS["base"], B=2, Q=600), seed=21, device=dev)
+    sh, lsi = inp["spatial_shapes"], inp["level_start_index"]
+    shared = inp["value_dpt_dist"][:, :, :1].contiguous()
+    packed = _ext.pack_shared_dist(shared, sh, lsi)
+    g = torch.Generator().manual_seed(1)
+    gwu = torch.randn(2, 600, 8, 1, generator=g).to(dev)
+    results = []
+    for extra in ((), (packed,)):
+        leaves = [x.clone().requires_grad_() for x in (inp["value"], shared, inp["sampling_locations"], inp["attention_weights"])]
+        out, wu = F.apply(leaves[0], leaves[1], sh, lsi, leaves[2], leaves[3], 64, *extra)
+        grads = torch.autograd.grad([out, wu], leaves, [inp["grad_output"], gwu])
+        results.append((out.detach(), wu.detach(), *grads))
+    plain = _ext.dfa3d_fused_forward(inp["value"], shared, sh, lsi, inp["sampling_locations"], inp["attention_weights"], 64,
+                                     need_depth_score=False, need_weight_update=True)
+    for r in results:
+        assert torch.equal(r[0], plain[0]) and torch.equal(r[1], plain[2])
+    for a, b in zip(results[0][2:], results[1][2:]):
+        torch.testing.assert_close(a, b, **F32_BWD)
+    one_bin = shared[..., :1].contiguous()
+    assert _ext.pack_shared_dist(one_bin, sh, lsi) is None and _ext.pack_shared_dist(shared.double(), sh, lsi) is None
+    with pytest.raises(RuntimeError, match="shared by all heads"):
+        _ext.dfa3d_fused_forward(inp["value"], inp["value_dpt_dist"], sh, lsi, inp["sampling_locations"],
+                                 inp["attention_weights"], 64, packed_dist=packed)

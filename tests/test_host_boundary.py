@@ -37,22 +37,22 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     null = ctypes.c_void_p(0)
     one = ctypes.c_void_p(256)          # never dereferenced: validation fails first
     # non-positive dimension
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 0, 10, 8, 32, 16, 2, 5, 4, 8, 0, None, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, null, 0, 10, 8, 32, 16, 2, 5, 4, 8, 0, None, null)
     assert rc == -1 and b"positive" in L.dfa3d_last_error()
     # unknown dtype
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 7, None, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 7, None, null)
     assert rc == -1 and b"dtype" in L.dfa3d_last_error()
     # too many levels
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 17, 5, 4, 8, 0, None, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, null, 1, 10, 8, 32, 16, 17, 5, 4, 8, 0, None, null)
     assert rc == -2 and b"levels" in L.dfa3d_last_error()
     # a batch element beyond 2^30 bytes
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 1 << 20, 8, 64, 16, 2, 5, 4, 8, 0, None, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, null, 1, 1 << 20, 8, 64, 16, 2, 5, 4, 8, 0, None, null)
     assert rc == -2 and b"2^30" in L.dfa3d_last_error()
     # NULL operand
-    rc = L.dfa3d_fused_forward(null, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 0, None, null)
+    rc = L.dfa3d_fused_forward(null, one, one, one, one, one, one, one, null, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 0, None, null)
     assert rc == -1 and b"NULL" in L.dfa3d_last_error()
     # a distribution for 3 of the 8 heads
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 3, 0, None, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, null, 1, 10, 8, 32, 16, 2, 5, 4, 3, 0, None, null)
     assert rc == -1 and b"dist_heads" in L.dfa3d_last_error()
     rc = L.dfa3d_wms_deform_attn_forward(one, one, 4, one, one, 2, one, one, one, 1, 10, 8, 32, 2, 5, 4, 0, None, null)
     assert rc == -1 and b"stride" in L.dfa3d_last_error()
@@ -72,10 +72,18 @@ def test_c_abi_rejects_bad_arguments_without_launching():
     assert L.dfa3d_fused_backward_workspace_bytes(*dims, 1, 0, None) > \
         L.dfa3d_fused_backward_workspace_bytes(*dims, 8, 0, None) > 0
     assert L.dfa3d_fused_backward_workspace_bytes(*dims, 8, 1, None) == 0    # fp64: direct kernels
+    # packed head-shared distribution: a bound from S and L (the level shapes live on the device); not for one bin / fp64
+    assert L.dfa3d_packed_dist_bytes(6, 30825, 64, 4, 0) == 6 * (2 * 30825 + 8) * 64 * 16
+    assert L.dfa3d_packed_dist_bytes(6, 30825, 64, 4, 2) == 6 * (2 * 30825 + 8) * 64 * 8
+    assert L.dfa3d_packed_dist_bytes(6, 30825, 1, 4, 0) == 0 and L.dfa3d_packed_dist_bytes(6, 30825, 64, 4, 1) == 0
+    rc = L.dfa3d_pack_dist(one, one, one, one, 16, 6, 30825, 64, 4, 0, null)
+    assert rc == -1 and b"are needed" in L.dfa3d_last_error()
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, one, 1, 10, 8, 32, 16, 2, 5, 4, 8, 0, None, null)
+    assert rc == -1 and b"packed_dist" in L.dfa3d_last_error()           # a packed table with a distribution per head
     # bfloat16 gradient buffers (DFA3D_BF16G = 3): fused backward only, C and D multiples of 4
     assert L.dfa3d_fused_backward_workspace_bytes(*dims, 8, 3, None) == L.dfa3d_fused_backward_workspace_bytes(*dims, 8, 2, None)
     assert L.dfa3d_fused_backward_workspace_bytes(6, 30825, 8, 32, 63, 4, 10000, 8, 8, 3, None) == 0
-    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 3, None, null)
+    rc = L.dfa3d_fused_forward(one, one, one, one, one, one, one, one, null, null, 1, 10, 8, 32, 16, 2, 5, 4, 8, 3, None, null)
     assert rc == -1 and b"DFA3D_BF16G" in L.dfa3d_last_error()
 
 
@@ -90,7 +98,7 @@ def test_launch_options_are_per_call_and_checked():
     def fwd(**fields):
         o = _lib.LaunchOptions(**fields)
         # value is NULL: a call that passes the option checks stops at the operand check
-        return L.dfa3d_fused_forward(null, one, one, one, one, one, one, one, null, *dims, 8, 0, ctypes.pointer(o), null)
+        return L.dfa3d_fused_forward(null, one, one, one, one, one, one, one, null, null, *dims, 8, 0, ctypes.pointer(o), null)
 
     for bad in (dict(iters=-1), dict(iters=65), dict(vec=3), dict(tile=7), dict(tile=6500), dict(block=128),
                 dict(pass_=32), dict(chunk=8), dict(reserved=1)):
