@@ -87,6 +87,14 @@ class MSDeformableAttention3D_DFA3D(nn.Module):
         depth = spatial_shape.new_full((*spatial_shape.shape[:-1], 1), depth_dim)
         return torch.cat([spatial_shape, depth], dim=-1).contiguous()
 
+    def pack_dist(self, value_dpt_dist, spatial_shapes, level_start_index):
+        """``value_dpt_dist`` (bs, keys, D) laid out for the operator's depth taps (``dfa3D._ext.pack_shared_dist``);
+        None where that is not offered.  Valid for as long as the distribution's values do not change."""
+        from .. import _ext
+        bs, keys, depth = value_dpt_dist.shape
+        dist = value_dpt_dist.reshape(bs, keys, 1, depth).to(self.value_proj.weight.dtype).contiguous()
+        return _ext.pack_shared_dist(dist, self.get_spatial_shape_3D(spatial_shapes, depth), level_start_index)
+
     def sampling_locations(self, query, reference_points, spatial_shapes_3D):
         """Normalised (x, y, z) of every sampling point, (bs, Q, heads, L, points, 3): the head's learned
         offsets, divided by the level's (W, H, D), around the query's Z-anchor reference points
@@ -109,12 +117,14 @@ class MSDeformableAttention3D_DFA3D(nn.Module):
 
     def forward(self, query, key=None, value=None, value_dpt_dist=None, identity=None, query_pos=None,
                 key_padding_mask=None, reference_points=None, spatial_shapes=None, level_start_index=None,
-                return_depth_score=False, **kwargs):
+                return_depth_score=False, packed_dist=None, **kwargs):
         """Arguments and results as spatial_cross_attention.py:428-583: ``query`` (bs, Q, embed_dims),
         ``value`` (bs, keys, embed_dims), ``value_dpt_dist`` (bs, keys, D), ``reference_points``
         (bs, Q, num_Z_anchors, 3) normalised, ``spatial_shapes`` (L, 2) as (h, w), ``level_start_index`` (L,).
         Returns ``(output (bs, Q, embed_dims), weight_update (bs, Q, heads, 1))``; with
-        ``return_depth_score=True`` a third result, the operator's depth scores."""
+        ``return_depth_score=True`` a third result, the operator's depth scores.  ``packed_dist``: what
+        ``self.pack_dist(value_dpt_dist, spatial_shapes, level_start_index)`` returned for this very distribution;
+        an encoder that runs several of these layers on one distribution packs once and hands it to each."""
         if value is None:
             value = query
         if query_pos is not None:
@@ -150,7 +160,7 @@ class MSDeformableAttention3D_DFA3D(nn.Module):
             output, depth_score = MultiScale3DDeformableAttnFunction_fp32.apply(*args)
             weight_update = (depth_score.mean(dim=-1) * attention_weights).flatten(-2).sum(dim=-1, keepdim=True)
         else:
-            output, weight_update = MultiScale3DDeformableAttnWeightUpdateFunction_fp32.apply(*args)
+            output, weight_update = MultiScale3DDeformableAttnWeightUpdateFunction_fp32.apply(*args, packed_dist)
         if not self.batch_first:
             output = output.permute(1, 0, 2)
         return (output, weight_update, depth_score) if return_depth_score else (output, weight_update)

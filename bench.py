@@ -215,6 +215,37 @@ def short_name(n):
     return n.replace("dfa3d::", "").replace("void ", "").replace("(anonymous namespace)::", "")[:92]
 
 
+def summarize_json(path):
+    """Text form of one JSON line this script printed (a --micro run or an operator run)."""
+    doc = json.load(open(path))
+    rel = os.path.relpath(path, ROOT)
+    out = []
+    if "xcd_map" in doc:
+        out += ["", f"## {rel}: {doc['device']}, {doc['compute_units']} CUs, plain copy {doc['copy_gbs']} GB/s (read + write)"]
+        for launch, rows in doc["xcd_map"].items():
+            diag = ", ".join(f"{r['on_diagonal']}/{r['blocks']}" for r in rows)
+            out.append(f"workgroup -> XCD, launch of {launch} (workgroups x threads): workgroups with XCD == id % 8: {diag}; "
+                       f"XCD of id % 8 = 0..7: {rows[0]['xcd_of_block_mod_8']}")
+        if "row_gather" in doc:
+            out += ["", "random whole-row gathers (row_bytes/16 lanes per row), by footprint the rows are drawn from",
+                    f"{'row_bytes':>9s} {'footprint_MiB':>13s} {'in_flight':>9s} {'TB/s':>7s} {'ps/row':>7s} {'clocks/row/CU':>13s}"]
+            out += [f"{r['row_bytes']:9d} {r['footprint_mib']:13d} {r['in_flight']:9d} {r['tb_per_s']:7.2f} {r['ps_per_row']:7.1f} "
+                    f"{r['clocks_per_row_per_cu']:13.2f}" for r in doc["row_gather"]]
+            out += ["", "random 8-byte loads, one per lane (64 different cache lines per wavefront instruction)",
+                    f"{'footprint_MiB':>13s} {'in_flight':>9s} {'G loads/s':>9s} {'ps/load':>7s} {'clocks/load/CU':>14s}"]
+            out += [f"{r['footprint_mib']:13d} {r['in_flight']:9d} {r['g_loads_per_s']:9.1f} {r['ps_per_load']:7.1f} "
+                    f"{r['clocks_per_load_per_cu']:14.2f}" for r in doc["pair_gather"]]
+            out += ["", "LDS atomics, lanes per clock per CU (2.4 GHz)"]
+            out += [f"{r['pattern']:32s} {r['lanes_per_clock_per_cu']:7.3f}" for r in doc["lds_atomics"]]
+    elif "kernels" in doc:
+        k = doc["kernels"]
+        out.append(f"{rel}: step {doc['ms_per_step']:.4f} ms, forward kernel {k['forward']['avg_ms']:.4f} ms, "
+                   + (f"binning {k['backward_binning']['avg_ms']:.4f} ms, tile kernel {k['backward_tile']['avg_ms']:.4f} ms "
+                      f"(min {k['backward_tile']['min_ms']:.4f}), " if "backward_tile" in k else "")
+                   + f"copy {doc['attainable_gbs']:.0f} GB/s")
+    return out
+
+
 def summarize(name, dirs, commands):
     """Per-kernel tables from rocprofv3's rocpd databases (kernel durations; counters per dispatch, averaged) as
     text under profiles/, and the HBM-side bytes of the operator's kernels (FETCH_SIZE / WRITE_SIZE, each scaled
@@ -223,6 +254,9 @@ def summarize(name, dirs, commands):
     import sqlite3
     lines = [f"# {c}" for c in commands]
     scale, raw, workload = {}, {}, None
+    for path in [d for d in dirs if d.endswith(".json")]:
+        lines += summarize_json(path)
+    dirs = [d for d in dirs if not d.endswith(".json")]
     cols = ("fwd_attention_kernel", "tile_backward_kernel", "bin_points_kernel<0>", "bin_points_kernel<1>",
             "stream_copy_kernel")
     for d in dirs:

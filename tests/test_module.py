@@ -132,3 +132,23 @@ def test_module_matches_restated_reference_forward_and_gradients(oracle, batch_f
     names = ["query", "value", "value_dpt_dist"] + [n for n, _ in m.named_parameters()]
     for n, g_, w_ in zip(names, got_grads, want_grads):
         torch.testing.assert_close(g_.cpu(), w_, msg=lambda s, n=n: f"grad {n}: {s}", **tol)
+
+
+@pytest.mark.gpu
+def test_module_with_a_distribution_packed_once_for_several_calls():
+    """float32 module: the packed distribution handed in (as an encoder with several layers on one distribution
+    would) gives the output and weight_update of the call that packs for itself, bit for bit, and gradients."""
+    dev = torch.device("cuda:0")
+    m = _randomise(_module(embed_dims=16, num_heads=2, num_levels=3, num_points=4)).to(dev)
+    query, value, dist, ref, shapes, lsi, go = (t.to(dev) if torch.is_tensor(t) else t for t in _inputs(dtype=torch.float32))
+    kw = dict(value=value, value_dpt_dist=dist, reference_points=ref, spatial_shapes=shapes, level_start_index=lsi)
+    packed = m.pack_dist(dist, shapes, lsi)
+    assert packed is not None
+    q = query.clone().requires_grad_()
+    out1, wu1 = m(q, **kw)
+    out2, wu2 = m(q, packed_dist=packed, **kw)
+    out3, wu3 = m(q, packed_dist=packed, **kw)             # the same packed tensor again
+    assert torch.equal(out1, out2) and torch.equal(wu1, wu2) and torch.equal(out2, out3)
+    g1, = torch.autograd.grad(out1, q, go, retain_graph=True)
+    g2, = torch.autograd.grad(out2, q, go)
+    torch.testing.assert_close(g1, g2, rtol=1e-5, atol=1e-6)
