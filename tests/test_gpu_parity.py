@@ -715,6 +715,19 @@ def test_more_tiles_than_the_block_histogram_holds(oracle):
     _compare(_gpu_one_stage(inp, dev), _oracle_one_stage(oracle, inp), F32_FWD, F32_BWD)
 
 
+@pytest.mark.parametrize("case", [dict(seed=57, B=1, C=4, M=2, Q=2000, P=4, D=2, levels=((400, 410), (3, 5))),
+                                  dict(seed=58, B=2, C=8, M=3, Q=5, P=2100, D=4, levels=((30, 41),)),
+                                  dict(seed=59, B=1, C=8, M=9, Q=3, P=700, D=3, levels=((9, 9), (20, 17), (5, 4)))],
+                         ids=["2600-tiles", "2100-points-per-unit", "2100-points-per-unit-3-levels"])
+def test_binning_fallbacks(oracle, case):
+    """Shapes the block-sorted binning kernels leave to the plain ones: more than 2048 tiles per (batch, head)
+    (counted in LDS by the plain kernels up to 8192 tiles), and more than 2048 sampling points per unit."""
+    dev = _dev()
+    t = tiny_case(dtype=torch.float32, **case)
+    inp = _as_inputs(t)
+    _compare(_gpu_one_stage(inp, dev), _oracle_one_stage(oracle, inp), F32_FWD, F32_BWD)
+
+
 def test_every_point_in_one_pixel_cell(oracle):
     """All sampling points in the same pixel cell and depth interval: one tile gets everything (several work
     items for one bin, every tile address contested).  Sums of 12 000 float32 terms, checked against the
