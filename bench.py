@@ -207,7 +207,7 @@ def micro(sections="all"):
 # rocprofv3 summaries
 # ------------------------------------------------------------------------------------------------
 KERNEL_KEYS = (("fwd_attention_kernel", "forward"), ("tile_backward_kernel", "backward_tile"),
-               ("bin_points_kernel<1>", "bin_fill"), ("bin_points_kernel<0>", "bin_count"))
+               ("bin_fill_sorted_kernel", "bin_fill"), ("bin_count_kernel", "bin_count"))
 
 
 def short_name(n):
@@ -257,7 +257,7 @@ def summarize(name, dirs, commands):
     for path in [d for d in dirs if d.endswith(".json")]:
         lines += summarize_json(path)
     dirs = [d for d in dirs if not d.endswith(".json")]
-    cols = ("fwd_attention_kernel", "tile_backward_kernel", "bin_points_kernel<0>", "bin_points_kernel<1>",
+    cols = ("fwd_attention_kernel", "tile_backward_kernel", "bin_count_kernel", "bin_fill_sorted_kernel",
             "stream_copy_kernel")
     for d in dirs:
         for db in sorted(glob.glob(os.path.join(d, "**", "*.db"), recursive=True)):
@@ -625,7 +625,7 @@ def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
         bin_ms, tile_ms = sum(bin_t) / len(bin_t), sum(tile_t) / len(tile_t)
         kernels["backward_tile"] = entry("tile_backward_kernel (all gradients, one launch)", tile_ms, min(tile_t), bwd_bytes,
                                          "backward_tile")
-        kernels["backward_binning"] = {"kernel": "plan_and_clear + bin_points<0> + bin_scan + bin_points<1> (4 launches)",
+        kernels["backward_binning"] = {"kernel": "plan_and_clear + bin_count + bin_scan + bin_fill_sorted (+ their plain forms, which step aside)",
                                        "avg_ms": round(bin_ms, 4), "min_ms": round(min(bin_t), 4)}
         dom = "backward_tile" if tile_ms >= fwd_ms else "forward"
     else:
