@@ -10,10 +10,13 @@
 // meet another one of the same pass at their address).
 //
 //   plan_and_clear_kernel       validates the level table, lays out the tiles (bins), clears counters
-//   bin_points_kernel<0>        points per bin (LDS histogram per block, one atomic per touched bin)
+//   bin_count_kernel            points per bin (LDS histogram per block, one atomic per touched bin)
 //   bin_scan_kernel             exclusive prefix over bins, work items (bin, chunk of its points)
-//   bin_points_kernel<1>        writes each point's index and record into its bin's segment; zero
+//   bin_fill_sorted_kernel      writes each point's index and record into its bin's segment, a block's points
+//                               sorted by bin in LDS first so that runs of records leave together; zero
 //                               gradients for points the operator skips
+//   bin_points_kernel<0>, <1>   count and fill for shapes the two above do not take (more than 2048 tiles per
+//                               (batch, head), more than 2048 points per unit): every record straight to its slot
 //   tile_backward_kernel        persistent workgroups pull work items from per-XCD queues; per item: LDS
 //                               tiles of (TY+1) x (TX+1) pixels (one-pixel halo to the right/bottom, so
 //                               all four corners of a point of this bin land in the tile), the phases

@@ -67,11 +67,15 @@ def parse():
 
 
 def sources_digest():
-    """SHA-256 over the kernel sources: what a traffic figure from the profiler is valid for."""
+    """SHA-256 over the kernel sources without their comments and blank space: what a traffic figure from the
+    profiler is valid for."""
     h = hashlib.sha256()
     for path in sorted(glob.glob(os.path.join(PKG, "csrc", "*.hip")) + glob.glob(os.path.join(PKG, "csrc", "*.h"))):
+        text = open(path, encoding="utf-8").read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        text = re.sub(r"//[^\n]*", "", text)
         h.update(os.path.basename(path).encode())
-        h.update(open(path, "rb").read())
+        h.update(" ".join(text.split()).encode())
     return h.hexdigest()
 
 
