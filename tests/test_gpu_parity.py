@@ -487,6 +487,56 @@ def test_launch_options_do_not_change_results(oracle, setting):
         _compare(_gpu_two_stage(inp, dev, sliced=False), want, F32_FWD, F32_BWD)
 
 
+def _random_case_with_options(seed):
+    """A wider draw than _random_case (channel counts up to 256, depth bins up to 128, up to 3000 queries on maps of
+    1 to 60 pixels a side, locations inside, around and in a corner of the map) with launch options drawn from
+    what the library accepts."""
+    import random
+    r = random.Random(seed)
+    L = r.randint(1, 5)
+    side = 60 if r.random() < 0.4 else 24
+    levels = tuple((r.randint(1, side), r.randint(1, side)) for _ in range(L))
+    case = dict(seed=seed, B=r.randint(1, 3), M=r.choice([1, 2, 3, 4, 5, 7, 8, 9, 16]),
+                C=r.choice([1, 2, 3, 4, 8, 12, 16, 20, 24, 32, 36, 40, 48, 64, 72, 96, 128, 160, 256]),
+                D=r.choice([1, 2, 3, 4, 7, 8, 16, 17, 32, 48, 64, 80, 112, 128]),
+                Q=r.choice([1, 2, 7, 33, 100, 257, 600, 1500, 3000]), P=r.randint(1, 9), levels=levels,
+                lo=r.choice([0.0, -0.2, 0.3]), hi=r.choice([1.0, 1.2, 0.6]))
+    points = case["B"] * case["Q"] * case["M"] * L * case["P"]
+    if points * case["C"] > 3e8 or points > 3e6:
+        case["Q"] = max(1, case["Q"] // 10)
+    opts = {}
+    if r.random() < 0.6:
+        for name, p, choices in (("tile", 0.5, [202, 203, 404, 408, 804, 808, 816, 1616, 302, 505]),
+                                 ("block", 0.3, [256, 512]), ("pass_", 0.3, [64, 128, 256]),
+                                 ("chunk", 0.3, [64, 100, 256, 1000, 4096]), ("vec", 0.3, [1, 2, 4, 8]),
+                                 ("iters", 0.2, [1, 2, 3, 5]), ("direct", 0.1, [1])):
+            if r.random() < p:
+                opts[name] = r.choice(choices)
+    return case, opts
+
+
+@pytest.mark.parametrize("seed", range(7000, 7048))
+def test_fp32_random_shapes_with_random_launch_options(oracle, seed):
+    """One-stage and two-stage paths on drawn shapes under drawn launch options.  Outputs, scores and per-point
+    gradients within the float32 gates plus 4e-6 of the tensor's largest element (dot products over up to 256
+    channels scaled by the map size); grad_value / grad_dist within the term-count bound of the float64 checker."""
+    from dfa3D import _lib
+    dev = _dev()
+    case, opts = _random_case_with_options(seed)
+    print("case", case, "options", opts, flush=True)
+    t = tiny_case(**case)
+    inp = {k: (v.float() if v.is_floating_point() else v) for k, v in _as_inputs(t).items()}
+    want = _oracle_one_stage(oracle, inp)
+    with _lib.launch_options(**opts):
+        results = (_gpu_one_stage(inp, dev), _gpu_two_stage(inp, dev, sliced=seed % 2 == 0))
+    for got in results:
+        for i, name in ((0, "output"), (1, "depth_score"), (4, "grad_loc"), (5, "grad_attn")):
+            tol = dict(F32_FWD if i < 2 else F32_BWD)
+            tol["atol"] += 4e-6 * want[i].abs().max().item()
+            torch.testing.assert_close(got[i], want[i], msg=lambda m, n=name: f"{n}: {m}", **tol)
+        _assert_sums_within_term_count_bound(oracle, inp, got[2], got[3])
+
+
 def test_fp32_base_shape_two_stage_matches_checker(oracle):
     from dfa3D.workloads import WORKLOADS, make_inputs
     dev = _dev()
