@@ -24,7 +24,7 @@ class Workload:
     P: int                      # sampling points per level
     M: int = 8                  # heads
     C: int = 32                 # channels per head
-    loc: str = "uniform"        # "uniform" in [lo, hi]^3 or "normal" clipped to [lo, hi]
+    loc: str = "uniform"        # "uniform" in [lo, hi]^3, "normal" clipped to [lo, hi], or "coherent" (see make_inputs)
     loc_lo: float = 0.0
     loc_hi: float = 1.0
     loc_mean: float = 0.5
@@ -82,12 +82,18 @@ WORKLOADS = {
     # the operands of the reference's own test (unittest_DFA3D.py:43-56): 112 depth bins, 9502 queries, attention
     # weights drawn from U[0,1) without normalisation
     "unittest": Workload("unittest", B=6, Q=9502, levels=_BASE_LEVELS, D=112, P=8, attn="rand"),
+    # base shape with the locations a trained model produces rather than uniformly random ones: the queries of a
+    # camera are BEV pillars in raster order, whose reference points project to a smooth pattern in the image, and
+    # the learned offsets move the points of a query by a few pixels around it
+    # (spatial_cross_attention.py:505-538: reference point + offset / (W, H, D))
+    "base_coherent": Workload("base_coherent", B=6, Q=10000, levels=_BASE_LEVELS, D=64, P=8, depth_sigma=2.0,
+                              loc="coherent", loc_std=0.02),
     # dense BEV grid, clustered locations
     "dense": Workload("dense", B=6, Q=40000, levels=_BASE_LEVELS, D=128, P=8, loc="normal",
                       loc_lo=-0.1, loc_hi=1.1, depth_sigma=2.0),
 }
 
-SEEDS = {"unit": 1, "small": 2, "base": 3, "base_peaky": 4, "dense": 5, "unittest": 6}
+SEEDS = {"unit": 1, "small": 2, "base": 3, "base_peaky": 4, "dense": 5, "unittest": 6, "base_coherent": 7}
 
 
 def scaled(w: Workload, B=None, Q=None, name=None) -> Workload:
@@ -114,6 +120,16 @@ def make_inputs(w: Workload, seed=None, dtype=torch.float32, device="cpu", grad_
     if w.loc == "normal":
         loc = torch.randn(B, Q, M, L, P, 3, generator=g, dtype=torch.float32) * w.loc_std + w.loc_mean
         loc.clamp_(w.loc_lo, w.loc_hi)
+    elif w.loc == "coherent":
+        # query q sits at cell (q // side, q % side) of a side x side raster over the image; its L*P points per head
+        # scatter around that cell's centre with standard deviation loc_std (x, y) and 0.2 around mid-depth (z)
+        side = max(1, int(round(Q ** 0.5)))
+        q = torch.arange(Q, dtype=torch.float32)
+        centre = torch.stack([((q % side) + 0.5) / side, (torch.div(q, side, rounding_mode="floor") % side + 0.5) / side,
+                              torch.full((Q,), 0.5)], -1)
+        spread = torch.tensor([w.loc_std, w.loc_std, 0.2])
+        # (not clipped: a point outside the image is outside the image, as in the model)
+        loc = torch.randn(B, Q, M, L, P, 3, generator=g, dtype=torch.float32) * spread + centre.view(1, Q, 1, 1, 1, 3)
     else:
         loc = torch.rand(B, Q, M, L, P, 3, generator=g, dtype=torch.float32) * (w.loc_hi - w.loc_lo) + w.loc_lo
     if w.attn == "rand":

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the DFA3D operator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload base|small|unit|dense|base_bf16|unittest]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload base|small|unit|dense|base_bf16|unittest|base_coherent]
     python bench.py --micro [xcd]                yardsticks of the machine (copy, bare gathers, LDS atomics, XCD map)
     python bench.py --summarize NAME DIR [DIR..] tables from rocprofv3 output directories -> profiles/NAME.txt
 

@@ -386,6 +386,25 @@ def test_fp32_workloads_match_checker(oracle, name):
     _compare(_gpu_one_stage(inp, dev), _oracle_one_stage(oracle, inp), F32_FWD, F32_BWD)
 
 
+@pytest.mark.parametrize("Q", [2500, 999])
+def test_fp32_model_like_locations_match_checker(oracle, Q):
+    """Locations as a model produces them (queries in raster order over the image, the points of a query within a
+    few pixels of each other): one query puts several points into the same tile and the same pixel, and the
+    binning kernels spread each block's queries over the whole range (999 queries: not a multiple of anything)."""
+    from dfa3D.workloads import WORKLOADS, make_inputs, scaled
+    dev = _dev()
+    inp = make_inputs(scaled(WORKLOADS["base_coherent"], B=2, Q=Q), seed=Q)
+    got = _gpu_one_stage(inp, dev)
+    want = _oracle_one_stage(oracle, inp)
+    for i in (0, 1, 4, 5):
+        torch.testing.assert_close(got[i], want[i], **(F32_FWD if i < 2 else F32_BWD))
+    _assert_sums_within_term_count_bound(oracle, inp, got[2], got[3])
+    got2 = _gpu_two_stage(inp, dev, sliced=False)
+    for i in (0, 1, 4, 5):
+        torch.testing.assert_close(got2[i], want[i], **(F32_FWD if i < 2 else F32_BWD))
+    _assert_sums_within_term_count_bound(oracle, inp, got2[2], got2[3])
+
+
 def _gpu_two_stage(inp, dev, sliced):
     """The reference's two-stage composition; `sliced` hands the 2-D stage (L,2) shapes and (…,2)
     locations as the reference does, otherwise the 3-wide tensors go in as they are."""
