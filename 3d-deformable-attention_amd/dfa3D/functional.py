@@ -178,7 +178,6 @@ class MultiScale3DDeformableAttnFunction(Function):
     def backward(ctx, grad_output, grad_depth_score):
         value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations, \
             attention_weights = ctx.saved_tensors
-        aux = _aux(value)
         if grad_output is None:
             grad_output = torch.zeros(value.shape[0], sampling_locations.shape[1], value.shape[2] * value.shape[3],
                                       dtype=value.dtype, device=value.device)
