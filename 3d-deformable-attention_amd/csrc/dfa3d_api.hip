@@ -29,7 +29,7 @@ int hip_result(hipError_t e, const char *what) {
 }
 
 // Launch options of one call, checked.  A NULL pointer stands for the defaults.
-int check_opts(const char *fn, const dfa3d_launch_options *o, dfa3d_launch_options *out) {
+int check_opts(const char *fn, const dfa3d_launch_options *o, dfa3d_launch_options *out, bool clear_ok = false) {
   dfa3d_launch_options r;
   memset(&r, 0, sizeof(r));
   if (o != nullptr) r = *o;
@@ -46,7 +46,10 @@ int check_opts(const char *fn, const dfa3d_launch_options *o, dfa3d_launch_optio
     return fail(DFA3D_EINVAL, "%s: options.pass must be 0, 64, 128 or 256", fn);
   if (r.chunk != 0 && (r.chunk < 64 || r.chunk > (1 << 20)))   // 64 = kMinChunk of the binned backward
     return fail(DFA3D_EINVAL, "%s: options.chunk must be 0 or in [64, 2^20]", fn);
-  if (r.reserved != 0) return fail(DFA3D_EINVAL, "%s: options.reserved must be 0", fn);
+  if (r.clear != 0 && r.clear != 1) return fail(DFA3D_EINVAL, "%s: options.clear must be 0 or 1", fn);
+  if (r.clear != 0 && !clear_ok)
+    return fail(DFA3D_EINVAL, "%s: options.clear is for the dfa3d_fused_backward calls only: this call's gradient "
+                "buffers must be zero on entry", fn);
   *out = r;
   return 0;
 }
@@ -60,7 +63,7 @@ std::atomic<int> g_stage{0};
 
 void apply_opts(dfa3d::BwdArgs &a, const dfa3d_launch_options &o) {
   a.iters = o.iters; a.vec_hint = o.vec; a.tile_hint = o.tile; a.block_hint = o.block; a.chunk_hint = o.chunk;
-  a.pass_hint = o.pass; a.event_binned = o.event_binned;
+  a.pass_hint = o.pass; a.event_binned = o.event_binned; a.clear_grads = o.clear;
 #ifdef DFA3D_EXPERIMENT
   a.diag = g_diag.load(std::memory_order_relaxed);
   a.stage = g_stage.load(std::memory_order_relaxed);
@@ -97,7 +100,7 @@ int check_dims(const char *fn, int B, int S, int M, int width, int L, int Q, int
 extern "C" {
 
 const char *dfa3d_last_error(void) { return g_err; }
-int dfa3d_abi_version(void) { return 8; }
+int dfa3d_abi_version(void) { return 9; }
 
 #ifdef DFA3D_EXPERIMENT
 int dfa3d_experiment_set(const char *name, int value) {
@@ -286,6 +289,19 @@ static dfa3d::BwdArgs fused_bwd_args(const void *value, const void *dist, const 
   return a;
 }
 
+// The fused backward on the direct kernels, which add every term straight into grad_value / grad_dist: with
+// options.clear the whole of both buffers is cleared first (float or double gradients here).
+static int direct_fused_backward(const char *fn, const dfa3d::BwdArgs &a, int dtype, int dist_heads, hipStream_t stream) {
+  if (a.clear_grads) {
+    const size_t elem = dtype == DFA3D_F64 ? 8 : 4;
+    if (hipError_t e = dfa3d::launch_zero_fill(a.grad_value, (size_t)a.B * a.S * a.M * a.C * elem, stream))
+      return hip_result(e, fn);
+    if (hipError_t e = dfa3d::launch_zero_fill(a.grad_dist, (size_t)a.B * a.S * dist_heads * a.D * elem, stream))
+      return hip_result(e, fn);
+  }
+  return hip_result(dfa3d::launch_backward(a, dtype, stream), fn);
+}
+
 size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, int L, int Q, int P, int dist_heads,
                                             int dtype, const dfa3d_launch_options *opts) {
   const char *fn = "dfa3d_fused_backward_workspace_bytes";
@@ -293,7 +309,7 @@ size_t dfa3d_fused_backward_workspace_bytes(int B, int S, int M, int C, int D, i
   const bool g16 = dtype == DFA3D_BF16G;
   if (g16) dtype = DFA3D_BF16;
   if (check_dims(fn, B, S, M, C, L, Q, P, dtype) || check_dims(fn, B, S, M, D, L, Q, P, dtype) ||
-      check_opts(fn, opts, &o))
+      check_opts(fn, opts, &o, true))
     return 0;
   if (o.direct) return 0;
   dfa3d::BwdArgs a = fused_bwd_args(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
@@ -315,7 +331,7 @@ int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *sha
   if (g16) dtype = DFA3D_BF16;
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
-  if (int rc = check_opts(fn, opts, &o)) return rc;
+  if (int rc = check_opts(fn, opts, &o, true)) return rc;
   if (dist_heads != M && dist_heads != 1) return fail(DFA3D_EINVAL, "%s: dist_heads must be M or 1", fn);
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
   REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
@@ -331,7 +347,7 @@ int dfa3d_fused_backward(const void *value, const void *dist, const int64_t *sha
   if (g16) return fail(DFA3D_EINVAL, "%s: DFA3D_BF16G (bfloat16 gradients) runs on the binned kernels only: pass a "
                        "workspace of dfa3d_fused_backward_workspace_bytes(..., DFA3D_BF16G, ...) bytes (0 = not offered "
                        "for these dimensions: use DFA3D_BF16 with float gradients)", fn);
-  return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
+  return direct_fused_backward(fn, a, dtype, dist_heads, (hipStream_t)stream);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -376,7 +392,7 @@ int dfa3d_fused_backward_static(const void *value, const void *dist, const int64
   if (g16) dtype = DFA3D_BF16;
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
   if (int rc = check_dims(fn, B, S, M, D, L, Q, P, dtype)) return rc;
-  if (int rc = check_opts(fn, opts, &o)) return rc;
+  if (int rc = check_opts(fn, opts, &o, true)) return rc;
   if (dist_heads != M && dist_heads != 1) return fail(DFA3D_EINVAL, "%s: dist_heads must be M or 1", fn);
   REQUIRE_PTR(fn, value); REQUIRE_PTR(fn, dist); REQUIRE_PTR(fn, shapes3); REQUIRE_PTR(fn, level_start);
   REQUIRE_PTR(fn, loc3); REQUIRE_PTR(fn, attn); REQUIRE_PTR(fn, grad_out); REQUIRE_PTR(fn, grad_value);
@@ -396,7 +412,7 @@ int dfa3d_fused_backward_static(const void *value, const void *dist, const int64
     if (e != hipErrorNotSupported) return hip_result(e, fn);
   }
   if (g16) return fail(DFA3D_EINVAL, "%s: DFA3D_BF16G is not offered for these dimensions", fn);
-  return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);   // no scratch needed at all
+  return direct_fused_backward(fn, a, dtype, dist_heads, (hipStream_t)stream);   // no scratch needed at all
 }
 
 static int check_rebatch(const char *fn, int bs, int cams, int max_len, int Nq, int E, int dtype) {

@@ -1214,6 +1214,77 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(float4 *__restrict__ dst
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256)
     dst[i] = make_float4(0, 0, 0, 0);
 }
+__global__ __launch_bounds__(64) void fill_zero_words_kernel(uint32_t *__restrict__ dst, size_t n) {
+  for (size_t i = threadIdx.x; i < n; i += 64) dst[i] = 0;
+}
+
+hipError_t launch_zero_fill(void *dst, size_t bytes, hipStream_t stream) {
+  if (dst == nullptr || (bytes & 3) != 0 || ((uintptr_t)dst & 3) != 0) return hipErrorInvalidValue;
+  char *p = static_cast<char *>(dst);
+  const size_t head = ((uintptr_t)p & 15) ? 16 - ((uintptr_t)p & 15) : 0;        // bytes before the first 16-byte boundary
+  const size_t lead = head < bytes ? head : bytes, body = (bytes - lead) & ~(size_t)15, tail = bytes - lead - body;
+  if (lead) hipLaunchKernelGGL(fill_zero_words_kernel, dim3(1), dim3(64), 0, stream, reinterpret_cast<uint32_t *>(p), lead / 4);
+  if (body) hipLaunchKernelGGL(fill_zero_kernel, dim3(2048), dim3(256), 0, stream, reinterpret_cast<float4 *>(p + lead), body / 16);
+  if (tail) hipLaunchKernelGGL(fill_zero_words_kernel, dim3(1), dim3(64), 0, stream, reinterpret_cast<uint32_t *>(p + lead + body), tail / 4);
+  return hipGetLastError();
+}
+
+// What the tile kernel adds to instead of storing, cleared for a caller that did not zero grad_value / grad_dist
+// (options.clear).  The tile kernel stores the rows of the pixels that lie inside a tile (not on its first row or
+// column, which are the halo of its upper and left neighbours) when that tile's points fit one work item and the
+// rows are whole 16-byte groups; every other row of the two tensors only ever receives atomic adds, or nothing:
+// pixels on tile rims, pixels of tiles without points or with several work items, keys outside every level.
+// A lane decides for one (batch, key, head) row; the wavefront then clears its 64 consecutive rows together, 16 bytes
+// per lane on consecutive addresses (the heads of a key share their fate, so whole lines go out).
+__device__ __forceinline__ void clear_rows_of_wave(char *base, size_t first_row, int row_bytes, bool clear_mine, int lane) {
+  char *dst = base + first_row * row_bytes;
+  if ((row_bytes & 15) == 0) {
+    const int n16 = row_bytes >> 4;
+    for (int c = lane; c < kWave * n16; c += kWave) {
+      const int r = c / n16;
+      if (__shfl((int)clear_mine, r, kWave)) *reinterpret_cast<uint4 *>(dst + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
+    }
+  } else {
+    const int n4 = row_bytes >> 2;
+    for (int c = lane; c < kWave * n4; c += kWave) {
+      const int r = c / n4;
+      if (__shfl((int)clear_mine, r, kWave)) *reinterpret_cast<uint32_t *>(dst + (size_t)c * 4) = 0;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void clear_unstored_kernel(BinWorkspace ws, char *__restrict__ grad_value, int value_row_bytes,
+                                                             char *__restrict__ grad_dist, int dist_row_bytes, int B, int S,
+                                                             int M, int L, int stores) {
+  const BinPlan &p = *ws.plan;
+  const int nb = p.bins_per_bm, TY = p.ty, TX = p.tx, ch = p.chunk;
+  const size_t rows = (size_t)B * S * M;
+  const int lane = threadIdx.x % kWave;
+  // every wavefront takes 64 consecutive rows per turn; all its lanes stay in the loop (shuffles)
+  for (size_t i0 = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) - lane; i0 < rows; i0 += (size_t)gridDim.x * blockDim.x) {
+    const size_t i = i0 + lane;
+    bool clear_mine = i < rows;
+    if (clear_mine && stores && nb > 0) {
+      const int m = (int)(i % M);
+      const size_t bs = i / M;
+      const int s = (int)(bs % S), b = (int)(bs / S);
+      for (int l = 0; l < L; ++l) {
+        const int local = s - p.start[l];
+        if (p.H[l] > 0 && local >= 0 && local < p.H[l] * p.W[l]) {
+          const int y = local / p.W[l], x = local - y * p.W[l];
+          if (y % TY != 0 && x % TX != 0) {
+            const int bin = slot_of(b, m, B, M) * nb + p.level_base[l] + (y / TY) * p.tiles_x[l] + x / TX;
+            const int c = ws.counts[bin];
+            clear_mine = !(c > 0 && c <= ch);                 // exactly one work item: it stores this row
+          }
+          break;
+        }
+      }
+    }
+    clear_rows_of_wave(grad_value, i0, value_row_bytes, clear_mine, lane);
+    if (grad_dist != nullptr) clear_rows_of_wave(grad_dist, i0, dist_row_bytes, clear_mine, lane);
+  }
+}
 
 // dst[r, :] = sum over heads m of src[r, m, :], rows of D floats, heads in order; dst is float, or bfloat16
 // when dst16 is set (then D is a multiple of 4)
@@ -1493,12 +1564,26 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
   const size_t need = workspace_bytes_for(a, kind, dtype);
   if (need == 0 || workspace == nullptr || workspace_bytes < need || ((uintptr_t)workspace & 255) != 0)
     return hipErrorNotSupported;
+  if (a.clear_grads) {
+    if (kind != 0) return hipErrorInvalidValue;            // the fused entry points only
+    // clear_unstored_kernel writes 16-byte groups where a row is made of them: buffers on 16-byte boundaries,
+    // or the direct kernels (which clear everything) take the call
+    if ((((uintptr_t)a.grad_value | (uintptr_t)a.grad_dist) & 15) != 0) return hipErrorNotSupported;
+  }
   const TileConfig cfg = tile_config_of(a, kind);
   const BinLayout lay = bin_layout(a, cfg.ty, cfg.tx);
   const BinWorkspace ws = carve_workspace(workspace, lay);
   float *gd_heads = shared_dist(a) ? reinterpret_cast<float *>(static_cast<char *>(workspace) + lay.gd_heads) : nullptr;
   if (a.stage == 0 || a.stage == 1) {
     if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, stream)) return e;
+  }
+  if (a.clear_grads) {
+    const int ge = a.grad_bf16 ? 2 : 4;
+    const size_t rows = (size_t)a.B * a.S * a.M;
+    const unsigned grid = (unsigned)((rows + 255) / 256 < 16384 ? (rows + 255) / 256 : 16384);
+    hipLaunchKernelGGL(clear_unstored_kernel, dim3(grid), dim3(256), 0, stream, ws, static_cast<char *>(a.grad_value),
+                       a.C * ge, gd_heads != nullptr ? nullptr : static_cast<char *>(a.grad_dist), a.D * ge, a.B, a.S, a.M,
+                       a.L, ((a.C | a.D) & 3) == 0 ? 1 : 0);
   }
   if (a.event_binned != nullptr) {
     if (hipError_t e = hipEventRecord((hipEvent_t)a.event_binned, stream)) return e;

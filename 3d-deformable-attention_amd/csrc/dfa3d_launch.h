@@ -67,6 +67,7 @@ struct BwdArgs {
   const void *grad_weight_update;    // gradient arriving at the forward's weight_update output, or nullptr
   int dist_heads;                    // as in FwdArgs; grad_dist has the same head count
   int grad_bf16;                     // grad_value / grad_dist are bfloat16 (binned fused backward on bfloat16 storage only)
+  int clear_grads;                   // grad_value / grad_dist hold anything on entry (fused backward only): clear what is added to
   int B, S, M, C, D, L, Q, P;
   int iters;
   int vec_hint;
@@ -96,6 +97,8 @@ hipError_t launch_depth_score_backward(const DepthScoreBwdArgs &a, int dtype, hi
 size_t binned_backward_workspace_bytes(const BwdArgs &a, int kind, int dtype);
 hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, size_t workspace_bytes,
                                   hipStream_t stream);
+// Zero fill by a kernel (no memset node: callers may capture the stream in a graph); bytes a multiple of 4.
+hipError_t launch_zero_fill(void *dst, size_t bytes, hipStream_t stream);
 size_t binned_depth_score_backward_workspace_bytes(const DepthScoreBwdArgs &d, int dtype, int tile_hint);
 hipError_t launch_depth_score_backward_binned(const DepthScoreBwdArgs &d, int dtype, void *workspace,
                                               size_t workspace_bytes, int tile_hint, int chunk_hint,

@@ -14,6 +14,8 @@ kernel each.
 Element types: float32 or float64 throughout, or bfloat16 storage (value, distributions,
 output, scores in bfloat16; locations, attention weights and every gradient buffer float32).
 """
+import contextlib
+
 import torch
 
 from . import _lib
@@ -377,11 +379,13 @@ def fused_backward_grad_dtype(value, value_dpt_dist, sampling_locations):
 
 def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
                          attention_weights, grad_output, grad_depth_score, grad_value, grad_value_dpt_dist,
-                         grad_sampling_loc, grad_attn_weight, im2col_step, grad_weight_update=None):
+                         grad_sampling_loc, grad_attn_weight, im2col_step, grad_weight_update=None, clear=False):
     """One-kernel DFA3D backward.  ``grad_depth_score`` and ``grad_weight_update`` (gradients arriving at the
     depth_score and weight_update outputs) may be None.  Accumulates into ``grad_value`` / ``grad_value_dpt_dist``
-    (pre-zeroed by the caller; float32 / float64, or both bfloat16 where ``fused_backward_grad_dtype`` says so);
-    overwrites ``grad_sampling_loc`` (…, 3) and ``grad_attn_weight``."""
+    (float32 / float64, or both bfloat16 where ``fused_backward_grad_dtype`` says so): pre-zeroed by the caller as
+    the reference's are, or, with ``clear=True``, holding anything (``torch.empty``): the call then clears what its
+    kernels add to rather than store, about a quarter of the two buffers on the tile kernels.  Overwrites
+    ``grad_sampling_loc`` (…, 3) and ``grad_attn_weight``."""
     named = dict(value=value, value_dpt_dist=value_dpt_dist, spatial_shapes=value_spatial_shapes,
                  level_start_index=value_level_start_index, sampling_loc=sampling_locations,
                  attn_weight=attention_weights, grad_output=grad_output, grad_value=grad_value,
@@ -412,18 +416,22 @@ def dfa3d_fused_backward(value, value_dpt_dist, value_spatial_shapes, value_leve
     _expect(grad_attn_weight, "grad_attn_weight", shape=(B, Q, M, L, P), dtype=aux)
     _step(B, im2col_step)
     if grad_output.numel() == 0:
+        if clear:
+            grad_value.zero_()
+            grad_value_dpt_dist.zero_()
         return
     code = _lib.DFA3D_BF16G if g16 else _lib.dtype_code(value)
-    # scratch for the binned (LDS-accumulating) kernels; 0 bytes means the direct kernel is used
-    ws_bytes = _lib.lib().dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2], code,
-                                                                _lib.options())
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
-    with torch.cuda.device(dev):
-        rc = _lib.lib().dfa3d_fused_backward(
-            _lib.ptr(value), _lib.ptr(value_dpt_dist), _lib.ptr(value_spatial_shapes),
-            _lib.ptr(value_level_start_index), _lib.ptr(sampling_locations), _lib.ptr(attention_weights),
-            _lib.ptr(grad_output), _lib.ptr(grad_depth_score), _lib.ptr(grad_weight_update), _lib.ptr(grad_value),
-            _lib.ptr(grad_value_dpt_dist), _lib.ptr(grad_sampling_loc), _lib.ptr(grad_attn_weight),
-            _lib.ptr(workspace), ws_bytes, B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2], code,
-            _lib.options(), _lib.stream_of(value))
+    with (_lib.launch_options(clear=1) if clear else contextlib.nullcontext()):
+        # scratch for the binned (LDS-accumulating) kernels; 0 bytes means the direct kernel is used
+        ws_bytes = _lib.lib().dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2],
+                                                                    code, _lib.options())
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
+        with torch.cuda.device(dev):
+            rc = _lib.lib().dfa3d_fused_backward(
+                _lib.ptr(value), _lib.ptr(value_dpt_dist), _lib.ptr(value_spatial_shapes),
+                _lib.ptr(value_level_start_index), _lib.ptr(sampling_locations), _lib.ptr(attention_weights),
+                _lib.ptr(grad_output), _lib.ptr(grad_depth_score), _lib.ptr(grad_weight_update), _lib.ptr(grad_value),
+                _lib.ptr(grad_value_dpt_dist), _lib.ptr(grad_sampling_loc), _lib.ptr(grad_attn_weight),
+                _lib.ptr(workspace), ws_bytes, B, S, M, C, D, L, Q, P, value_dpt_dist.shape[2], code,
+                _lib.options(), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_fused_backward")

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdfa3d_hip.so")
 
 DFA3D_F32, DFA3D_F64, DFA3D_BF16, DFA3D_BF16G = 0, 1, 2, 3
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _P, _I = ctypes.c_void_p, ctypes.c_int
 _DIMS7 = [_I] * 7      # B S M (C|D) L Q P
@@ -24,7 +24,7 @@ _DIMS8 = [_I] * 8      # B S M C D L Q P
 class LaunchOptions(ctypes.Structure):
     """dfa3d_launch_options of include/dfa3d.h: how one call is laid out on the machine (never what it computes)."""
     _fields_ = [("iters", _I), ("vec", _I), ("direct", _I), ("tile", _I), ("block", _I), ("pass_", _I), ("chunk", _I),
-                ("reserved", _I), ("event_binned", _P)]
+                ("clear", _I), ("event_binned", _P)]
 
 
 _O = ctypes.POINTER(LaunchOptions)
@@ -97,7 +97,7 @@ def launch_options(**fields):
     for k, v in fields.items():
         if k == "pass":
             k = "pass_"
-        if k not in dict(LaunchOptions._fields_) or k == "reserved":
+        if k not in dict(LaunchOptions._fields_):
             raise TypeError(f"unknown launch option {k!r}")
         merged[k] = v
     saved = getattr(_tls, "fields", None)

@@ -182,15 +182,17 @@ class MultiScale3DDeformableAttnFunction(Function):
             grad_output = torch.zeros(value.shape[0], sampling_locations.shape[1], value.shape[2] * value.shape[3],
                                       dtype=value.dtype, device=value.device)
         gdt = _ext.fused_backward_grad_dtype(value, value_dpt_dist, sampling_locations)
-        grad_value = torch.zeros(value.shape, dtype=gdt, device=value.device)
-        grad_value_dpt_dist = torch.zeros(value_dpt_dist.shape, dtype=gdt, device=value.device)
+        # not zeroed here: the call clears the part of the two buffers that its kernels add to (clear=True)
+        grad_value = torch.empty(value.shape, dtype=gdt, device=value.device)
+        grad_value_dpt_dist = torch.empty(value_dpt_dist.shape, dtype=gdt, device=value.device)
         grad_sampling_loc = torch.empty_like(sampling_locations)
         grad_attn_weight = torch.empty_like(attention_weights)
         _ext.dfa3d_fused_backward(
             value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
             attention_weights, _grad_in(grad_output, value.dtype),
             None if grad_depth_score is None else _grad_in(grad_depth_score, value.dtype),
-            grad_value, grad_value_dpt_dist, grad_sampling_loc, grad_attn_weight, im2col_step=ctx.im2col_step)
+            grad_value, grad_value_dpt_dist, grad_sampling_loc, grad_attn_weight, im2col_step=ctx.im2col_step,
+            clear=True)
         return grad_value.to(value.dtype), grad_value_dpt_dist.to(value_dpt_dist.dtype), None, None, \
             grad_sampling_loc, grad_attn_weight, None
 
@@ -233,15 +235,16 @@ class MultiScale3DDeformableAttnWeightUpdateFunction(Function):
             grad_output = torch.zeros(value.shape[0], sampling_locations.shape[1], value.shape[2] * value.shape[3],
                                       dtype=value.dtype, device=value.device)
         gdt = _ext.fused_backward_grad_dtype(value, value_dpt_dist, sampling_locations)
-        grad_value = torch.zeros(value.shape, dtype=gdt, device=value.device)
-        grad_value_dpt_dist = torch.zeros(value_dpt_dist.shape, dtype=gdt, device=value.device)
+        grad_value = torch.empty(value.shape, dtype=gdt, device=value.device)
+        grad_value_dpt_dist = torch.empty(value_dpt_dist.shape, dtype=gdt, device=value.device)
         grad_sampling_loc = torch.empty_like(sampling_locations)
         grad_attn_weight = torch.empty_like(attention_weights)
         _ext.dfa3d_fused_backward(
             value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
             attention_weights, _grad_in(grad_output, value.dtype), None,
             grad_value, grad_value_dpt_dist, grad_sampling_loc, grad_attn_weight, im2col_step=ctx.im2col_step,
-            grad_weight_update=None if grad_weight_update is None else _grad_in(grad_weight_update, aux))
+            grad_weight_update=None if grad_weight_update is None else _grad_in(grad_weight_update, aux),
+            clear=True)
         # one gradient per forward argument: seven, or eight when the packed distribution was passed in
         return (grad_value.to(value.dtype), grad_value_dpt_dist.to(value_dpt_dist.dtype), None, None,
                 grad_sampling_loc, grad_attn_weight, None, None)

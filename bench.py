@@ -10,7 +10,9 @@ A step is one forward + backward of the one-stage autograd Function
 BEVFormer-shaped operands already resident in HBM.  Prints ONE JSON line:
 
   metric/value   sampled points (B*Q*M*L*P) per second of forward+backward, whole job
-  ms_per_step    forward+backward through autograd (includes its allocations and zero fills)
+  ms_per_step    forward+backward through autograd (includes its allocations; the backward call clears the part of
+                 the gradient buffers that its kernels add to: grad_zero_fill_ms, what zeroing both buffers in
+                 full takes, is reported beside it and is no part of a step)
   kernels        launch durations measured with events on the launch stream: the forward kernel, the
                  backward's binning kernels (as a group) and its tile kernel (the library records an event
                  between the two groups of the SAME call), with the algorithmic GB/s (each operand read once,
@@ -211,7 +213,8 @@ def micro(sections="all"):
 # rocprofv3 summaries
 # ------------------------------------------------------------------------------------------------
 KERNEL_KEYS = (("fwd_attention_kernel", "forward"), ("tile_backward_kernel", "backward_tile"),
-               ("bin_fill_sorted_kernel", "bin_fill"), ("bin_count_kernel", "bin_count"))
+               ("bin_fill_sorted_kernel", "bin_fill"), ("bin_count_kernel", "bin_count"),
+               ("clear_unstored_kernel", "clear"))
 
 
 def short_name(n):
@@ -575,11 +578,17 @@ def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
     mid_handle = mid.cuda_event
     assert mid_handle, "torch did not create the event"
 
+    user_fields = dict(user_options)
+    if "pass" in user_fields:
+        user_fields["pass_"] = user_fields.pop("pass")
+    # as the autograd Function calls it: gradient buffers not zeroed, the call clears what its kernels add to
+    default_opts = ctypes.pointer(_lib.LaunchOptions(clear=1, **user_fields))
+
     def backward_call(opts=None):
         _lib.check(L_.dfa3d_fused_backward(
             _lib.ptr(vd), _lib.ptr(dd), _lib.ptr(shapes), _lib.ptr(lsi), _lib.ptr(ld), _lib.ptr(ad), _lib.ptr(go), None,
             None, _lib.ptr(gv), _lib.ptr(gd), _lib.ptr(gl), _lib.ptr(ga), _lib.ptr(ws) if ws_bytes else None, ws_bytes,
-            B, S, M, C, D, L, Q, P, dist.shape[2], code, opts if opts is not None else _lib.options(), stream),
+            B, S, M, C, D, L, Q, P, dist.shape[2], code, opts if opts is not None else default_opts, stream),
             "dfa3d_fused_backward")
 
     def zero():
@@ -587,7 +596,7 @@ def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
         gd.zero_()
 
     fwd_ms, fwd_best = event_time(lambda: _ext.dfa3d_fused_forward(vd, dd, shapes, lsi, ld, ad, 64), a.kernel_reps)
-    bwd_all_ms, bwd_all_best = event_time(backward_call, a.kernel_reps, prep=zero)
+    bwd_all_ms, bwd_all_best = event_time(backward_call, a.kernel_reps)
     fill_ms, _ = event_time(zero, a.kernel_reps)
     traffic, traffic_note = ({}, "launch options given: recorded traffic does not apply") if user_options \
         else recorded_traffic(a.workload)
@@ -612,13 +621,9 @@ def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
     if ws_bytes:
         # the two parts of the SAME backward call: [start .. event recorded by the library] = binning kernels,
         # [that event .. end] = tile kernel (plus the head sum for a shared distribution)
-        fields = dict(user_options)
-        if "pass" in fields:
-            fields["pass_"] = fields.pop("pass")
-        opts = ctypes.pointer(_lib.LaunchOptions(event_binned=mid_handle, **fields))
+        opts = ctypes.pointer(_lib.LaunchOptions(event_binned=mid_handle, clear=1, **user_fields))
         bin_t, tile_t = [], []
         for _ in range(a.kernel_reps):
-            zero()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             backward_call(opts)
@@ -629,7 +634,7 @@ def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
         bin_ms, tile_ms = sum(bin_t) / len(bin_t), sum(tile_t) / len(tile_t)
         kernels["backward_tile"] = entry("tile_backward_kernel (all gradients, one launch)", tile_ms, min(tile_t), bwd_bytes,
                                          "backward_tile")
-        kernels["backward_binning"] = {"kernel": "plan_and_clear + bin_count + bin_scan + bin_fill_sorted (+ their plain forms, which step aside)",
+        kernels["backward_binning"] = {"kernel": "plan_and_clear + bin_count + bin_scan + bin_fill_sorted (+ their plain forms, which step aside) + clear_unstored",
                                        "avg_ms": round(bin_ms, 4), "min_ms": round(min(bin_t), 4)}
         dom = "backward_tile" if tile_ms >= fwd_ms else "forward"
     else:

@@ -53,8 +53,8 @@ extern "C" {
 #define DFA3D_MAX_LEVELS 16
 
 /* Launch options of ONE call.  NULL, or a zero-filled structure, means the defaults.  They choose how the
- * work is laid out on the machine and never what is computed: results agree up to floating-point
- * summation order of grad_value / grad_dist, whatever the values. */
+ * work is laid out on the machine (and, `clear`, who zeroes two output buffers) and never what is computed:
+ * results agree up to floating-point summation order of grad_value / grad_dist, whatever the values. */
 typedef struct dfa3d_launch_options {
   int iters;    /* groups of units each wavefront walks through; 0 = 1, at most 64 */
   int vec;      /* channels per lane in the row gathers: 0 = automatic, 1, 2 or 4 (8: tile kernels only) */
@@ -63,7 +63,10 @@ typedef struct dfa3d_launch_options {
   int block;    /* binned backward: threads per tile workgroup, 256 or 0/512 */
   int pass;     /* binned backward: points a tile workgroup takes per pass, 64, 128 or 256; 0 = automatic */
   int chunk;    /* binned backward: points of one tile handled by one work item, 0 = 4096 */
-  int reserved; /* must be 0 */
+  int clear;    /* dfa3d_fused_backward / dfa3d_fused_backward_static only (0 elsewhere): non-zero = grad_value and
+                 * grad_dist may hold anything on entry, the call clears what its kernels add to instead of
+                 * storing (a quarter of the buffers with the tile kernel, all of them otherwise); 0 = they are
+                 * zero on entry, as the reference's caller makes them */
   void *event_binned;   /* a hipEvent_t, or NULL: a binned backward records it on `stream` between its binning
                          * kernels and its tile kernel, so that a profiler can time the two parts of the call */
 } dfa3d_launch_options;
@@ -162,8 +165,9 @@ int dfa3d_pack_dist(const void *dist, const int64_t *shapes3, const int64_t *lev
  * read back.  `grad_score_in` (B,Q,M,L,P,4) and `grad_weight_update` (B,Q,M; float / double as
  * above), either of which may be NULL, are incoming gradients with respect to the `score` and
  * `weight_update` outputs and are chained into grad_dist, grad_attn and the z gradient.
- * `grad_value` (B,S,M,C) and `grad_dist` (B,S,dist_heads,D) must be zero on entry and hold the
- * gradients on return; `grad_loc3` and `grad_attn` are overwritten.
+ * `grad_value` (B,S,M,C) and `grad_dist` (B,S,dist_heads,D) must be zero on entry, as the reference's are,
+ * unless options.clear is set (then they may hold anything: the call clears what it does not overwrite),
+ * and hold the gradients on return; `grad_loc3` and `grad_attn` are overwritten.
  *
  * `workspace` (may be NULL) is caller-owned scratch device memory, 256-byte aligned, of at least
  * dfa3d_fused_backward_workspace_bytes(...) bytes, whose contents need not be preserved or

@@ -506,6 +506,72 @@ def test_launch_options_do_not_change_results(oracle, setting):
         _compare(_gpu_two_stage(inp, dev, sliced=False), want, F32_FWD, F32_BWD)
 
 
+@pytest.mark.parametrize("variant", ["tiles", "many-items", "odd-channels", "direct", "fp64", "shared", "bf16", "gap",
+                                     "static"])
+def test_gradient_buffers_that_were_not_zeroed(variant):
+    """options.clear: grad_value / grad_dist handed over full of NaN come back equal to what the call writes into
+    zeroed buffers, on the tile kernels (one work item per tile, several, tiles without points, rows that are
+    no whole 16-byte groups, keys that belong to no level), on the direct kernels, for a distribution shared by the
+    heads, for bfloat16 gradient buffers and through the entry point with the built-in scratch."""
+    import ctypes
+    from dfa3D import _ext, _lib
+    dev = _dev()
+    kw = dict(seed=300, B=2, M=8, C=32, D=16, Q=400, P=4, levels=((37, 52), (19, 26), (5, 3)), dtype=torch.float32)
+    opts = {}
+    if variant == "many-items":
+        opts = dict(chunk=64)
+    elif variant == "odd-channels":
+        kw.update(C=6, D=5)
+    elif variant == "direct":
+        opts = dict(direct=1)
+    elif variant == "fp64":
+        kw.update(dtype=torch.float64, Q=60)
+    t = tiny_case(**kw)
+    t["loc"][:, :, :, 0] = t["loc"][:, :, :, 0] * 0.3            # level 0: most tiles stay without points
+    value, dist, loc, attn, go = [t[k].to(dev) for k in ("value", "dist", "loc", "attn", "grad_out")]
+    shapes3, lsi = t["shapes3"].to(dev), t["lsi"].to(dev)
+    if variant == "gap":                                         # seven keys between the levels belong to no level
+        cut = int(lsi[1])
+        pad = lambda x: torch.cat([x[:, :cut], torch.randn_like(x[:, :7]), x[:, cut:]], 1).contiguous()
+        value, dist = pad(value), pad(dist)
+        lsi = lsi.clone()
+        lsi[1:] += 7
+    if variant == "shared":
+        dist = dist[:, :, :1].contiguous()
+    gdt = value.dtype
+    if variant == "bf16":
+        value, dist, go = value.bfloat16(), dist.bfloat16(), go.bfloat16()
+        gdt = _ext.fused_backward_grad_dtype(value, dist, loc)
+        assert gdt == torch.bfloat16
+
+    def run(fill, clear):
+        gv = torch.full(value.shape, fill, dtype=gdt, device=dev)
+        gd = torch.full(dist.shape, fill, dtype=gdt, device=dev)
+        gl, ga = torch.empty_like(loc), torch.empty_like(attn)
+        with _lib.launch_options(**opts):
+            if variant == "static":
+                B, S, M, C = value.shape
+                o = ctypes.pointer(_lib.LaunchOptions(clear=1 if clear else 0))
+                rc = _lib.lib().dfa3d_fused_backward_static(
+                    _lib.ptr(value), _lib.ptr(dist), _lib.ptr(shapes3), _lib.ptr(lsi), _lib.ptr(loc), _lib.ptr(attn),
+                    _lib.ptr(go), None, None, _lib.ptr(gv), _lib.ptr(gd), _lib.ptr(gl), _lib.ptr(ga), B, S, M, C,
+                    dist.shape[3], loc.shape[3], loc.shape[1], loc.shape[4], dist.shape[2], _lib.dtype_code(value), o,
+                    _lib.stream_of(value))
+                _lib.check(rc, "dfa3d_fused_backward_static")
+            else:
+                _ext.dfa3d_fused_backward(value, dist, shapes3, lsi, loc, attn, go, None, gv, gd, gl, ga, 64, clear=clear)
+        torch.cuda.synchronize()
+        return gv.float().cpu(), gd.float().cpu()
+
+    want_gv, want_gd = run(0.0, False)
+    got_gv, got_gd = run(float("nan"), True)
+    assert torch.isfinite(got_gv).all() and torch.isfinite(got_gd).all()
+    tol = dict(rtol=2e-2, atol=2e-2) if variant == "bf16" else dict(rtol=1e-5, atol=1e-5)    # order of the atomic adds
+    torch.testing.assert_close(got_gv, want_gv, **tol)
+    torch.testing.assert_close(got_gd, want_gd, **tol)
+    assert want_gv.abs().sum() > 0 and want_gd.abs().sum() > 0
+
+
 def _random_case_with_options(seed):
     """A wider draw than _random_case (channel counts up to 256, depth bins up to 128, up to 3000 queries on maps of
     1 to 60 pixels a side, locations inside, around and in a corner of the map) with launch options drawn from

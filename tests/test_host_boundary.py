@@ -101,12 +101,14 @@ def test_launch_options_are_per_call_and_checked():
         return L.dfa3d_fused_forward(null, one, one, one, one, one, one, one, null, null, *dims, 8, 0, ctypes.pointer(o), null)
 
     for bad in (dict(iters=-1), dict(iters=65), dict(vec=3), dict(tile=7), dict(tile=6500), dict(block=128),
-                dict(pass_=32), dict(chunk=8), dict(reserved=1)):
+                dict(pass_=32), dict(chunk=8), dict(clear=2), dict(clear=1)):   # clear: the fused backward calls only
         assert fwd(**bad) == -1 and b"options." in L.dfa3d_last_error(), bad
     assert fwd(iters=2, vec=4, tile=808, block=256, pass_=128, chunk=1024) == -1 and b"NULL" in L.dfa3d_last_error()
     big = (6, 30825, 8, 32, 64, 4, 10000, 8)
     assert L.dfa3d_fused_backward_workspace_bytes(*big, 8, 0, ctypes.pointer(_lib.LaunchOptions(direct=1))) == 0
     assert L.dfa3d_fused_backward_workspace_bytes(*big, 8, 0, ctypes.pointer(_lib.LaunchOptions(vec=3))) == 0
+    assert L.dfa3d_fused_backward_workspace_bytes(*big, 8, 0, ctypes.pointer(_lib.LaunchOptions(clear=1))) == \
+        L.dfa3d_fused_backward_workspace_bytes(*big, 8, 0, None)
     assert L.dfa3d_fused_backward_workspace_bytes(*big, 8, 0, ctypes.pointer(_lib.LaunchOptions(tile=404))) > \
         L.dfa3d_fused_backward_workspace_bytes(*big, 8, 0, None)            # more, smaller tiles: more counters
     assert not hasattr(L, "dfa3d_set_tunable") and not hasattr(L, "dfa3d_stream_copy")
