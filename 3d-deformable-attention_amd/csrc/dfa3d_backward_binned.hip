@@ -11,7 +11,8 @@
 //
 //   plan_and_clear_kernel       validates the level table, lays out the tiles (bins), clears counters
 //   bin_count_kernel            points per bin (LDS histogram per block, one atomic per touched bin)
-//   bin_scan_kernel             exclusive prefix over bins, work items (bin, chunk of its points)
+//   bin_scan_kernel             exclusive prefix over bins, work items (bin, chunk of its points); its further
+//                               blocks clear gradient rows for callers that did not zero them (options.clear)
 //   bin_fill_sorted_kernel      writes each point's index and record into its bin's segment, a block's points
 //                               sorted by bin in LDS first so that runs of records leave together; zero
 //                               gradients for points the operator skips
@@ -400,7 +401,76 @@ __global__ __launch_bounds__(kFillThreads) void bin_fill_sorted_kernel(
   }
 }
 
-__global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws) {
+// What the tile kernel adds to instead of storing, cleared for a caller that did not zero grad_value / grad_dist
+// (options.clear).  The tile kernel stores the rows of the pixels that lie inside a tile (not on its first row or
+// column, which are the halo of its upper and left neighbours) when that tile's points fit one work item and the
+// rows are whole 16-byte groups; every other row of the two tensors only ever receives atomic adds, or nothing:
+// pixels on tile rims, pixels of tiles without points or with several work items, keys outside every level.
+// A lane decides for one (batch, key, head) row; the wavefront then clears its 64 consecutive rows together, 16 bytes
+// per lane on consecutive addresses (the heads of a key share their fate, so whole lines go out).
+__device__ __forceinline__ void clear_rows_of_wave(char *base, size_t first_row, int row_bytes, bool clear_mine, int lane) {
+  char *dst = base + first_row * row_bytes;
+  if ((row_bytes & 15) == 0) {
+    const int n16 = row_bytes >> 4;
+    for (int c = lane; c < kWave * n16; c += kWave) {
+      const int r = c / n16;
+      if (__shfl((int)clear_mine, r, kWave)) *reinterpret_cast<uint4 *>(dst + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
+    }
+  } else {
+    const int n4 = row_bytes >> 2;
+    for (int c = lane; c < kWave * n4; c += kWave) {
+      const int r = c / n4;
+      if (__shfl((int)clear_mine, r, kWave)) *reinterpret_cast<uint32_t *>(dst + (size_t)c * 4) = 0;
+    }
+  }
+}
+
+struct ClearArgs {
+  char *grad_value, *grad_dist;     // grad_value == nullptr: nothing to clear; grad_dist == nullptr: not that one
+  int value_row_bytes, dist_row_bytes, B, S, M, L, stores;
+};
+__device__ __forceinline__ void clear_unstored(const BinWorkspace &ws, const ClearArgs &ca, unsigned block, unsigned n_blocks) {
+  char *grad_value = ca.grad_value, *grad_dist = ca.grad_dist;
+  const int value_row_bytes = ca.value_row_bytes, dist_row_bytes = ca.dist_row_bytes;
+  const int B = ca.B, S = ca.S, M = ca.M, L = ca.L, stores = ca.stores;
+  const BinPlan &p = *ws.plan;
+  const int nb = p.bins_per_bm, TY = p.ty, TX = p.tx, ch = p.chunk;
+  const size_t rows = (size_t)B * S * M;
+  const int lane = threadIdx.x % kWave;
+  // every wavefront takes 64 consecutive rows per turn; all its lanes stay in the loop (shuffles)
+  for (size_t i0 = ((size_t)block * blockDim.x + threadIdx.x) - lane; i0 < rows; i0 += (size_t)n_blocks * blockDim.x) {
+    const size_t i = i0 + lane;
+    bool clear_mine = i < rows;
+    if (clear_mine && stores && nb > 0) {
+      const int m = (int)(i % M);
+      const size_t bs = i / M;
+      const int s = (int)(bs % S), b = (int)(bs / S);
+      for (int l = 0; l < L; ++l) {
+        const int local = s - p.start[l];
+        if (p.H[l] > 0 && local >= 0 && local < p.H[l] * p.W[l]) {
+          const int y = local / p.W[l], x = local - y * p.W[l];
+          if (y % TY != 0 && x % TX != 0) {
+            const int bin = slot_of(b, m, B, M) * nb + p.level_base[l] + (y / TY) * p.tiles_x[l] + x / TX;
+            const int c = ws.counts[bin];
+            clear_mine = !(c > 0 && c <= ch);                 // exactly one work item: it stores this row
+          }
+          break;
+        }
+      }
+    }
+    clear_rows_of_wave(grad_value, i0, value_row_bytes, clear_mine, lane);
+    if (grad_dist != nullptr) clear_rows_of_wave(grad_dist, i0, dist_row_bytes, clear_mine, lane);
+  }
+}
+
+// Block 0 scans; further blocks, if any, clear the gradient rows that need it meanwhile (both only read the
+// counts: the scan is one workgroup's work and would leave the rest of the GPU idle).
+__global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws, ClearArgs ca) {
+  if (blockIdx.x > 0) {
+    clear_unstored(ws, ca, blockIdx.x - 1, gridDim.x - 1);
+    return;
+  }
+
   // One workgroup walks the bins 4096 at a time: four consecutive bins per thread (their loads are
   // independent, so a round costs one memory latency), a workgroup-wide exclusive scan of points and of
   // work items, and a running carry.
@@ -1229,63 +1299,6 @@ hipError_t launch_zero_fill(void *dst, size_t bytes, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// What the tile kernel adds to instead of storing, cleared for a caller that did not zero grad_value / grad_dist
-// (options.clear).  The tile kernel stores the rows of the pixels that lie inside a tile (not on its first row or
-// column, which are the halo of its upper and left neighbours) when that tile's points fit one work item and the
-// rows are whole 16-byte groups; every other row of the two tensors only ever receives atomic adds, or nothing:
-// pixels on tile rims, pixels of tiles without points or with several work items, keys outside every level.
-// A lane decides for one (batch, key, head) row; the wavefront then clears its 64 consecutive rows together, 16 bytes
-// per lane on consecutive addresses (the heads of a key share their fate, so whole lines go out).
-__device__ __forceinline__ void clear_rows_of_wave(char *base, size_t first_row, int row_bytes, bool clear_mine, int lane) {
-  char *dst = base + first_row * row_bytes;
-  if ((row_bytes & 15) == 0) {
-    const int n16 = row_bytes >> 4;
-    for (int c = lane; c < kWave * n16; c += kWave) {
-      const int r = c / n16;
-      if (__shfl((int)clear_mine, r, kWave)) *reinterpret_cast<uint4 *>(dst + (size_t)c * 16) = make_uint4(0, 0, 0, 0);
-    }
-  } else {
-    const int n4 = row_bytes >> 2;
-    for (int c = lane; c < kWave * n4; c += kWave) {
-      const int r = c / n4;
-      if (__shfl((int)clear_mine, r, kWave)) *reinterpret_cast<uint32_t *>(dst + (size_t)c * 4) = 0;
-    }
-  }
-}
-
-__global__ __launch_bounds__(256) void clear_unstored_kernel(BinWorkspace ws, char *__restrict__ grad_value, int value_row_bytes,
-                                                             char *__restrict__ grad_dist, int dist_row_bytes, int B, int S,
-                                                             int M, int L, int stores) {
-  const BinPlan &p = *ws.plan;
-  const int nb = p.bins_per_bm, TY = p.ty, TX = p.tx, ch = p.chunk;
-  const size_t rows = (size_t)B * S * M;
-  const int lane = threadIdx.x % kWave;
-  // every wavefront takes 64 consecutive rows per turn; all its lanes stay in the loop (shuffles)
-  for (size_t i0 = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) - lane; i0 < rows; i0 += (size_t)gridDim.x * blockDim.x) {
-    const size_t i = i0 + lane;
-    bool clear_mine = i < rows;
-    if (clear_mine && stores && nb > 0) {
-      const int m = (int)(i % M);
-      const size_t bs = i / M;
-      const int s = (int)(bs % S), b = (int)(bs / S);
-      for (int l = 0; l < L; ++l) {
-        const int local = s - p.start[l];
-        if (p.H[l] > 0 && local >= 0 && local < p.H[l] * p.W[l]) {
-          const int y = local / p.W[l], x = local - y * p.W[l];
-          if (y % TY != 0 && x % TX != 0) {
-            const int bin = slot_of(b, m, B, M) * nb + p.level_base[l] + (y / TY) * p.tiles_x[l] + x / TX;
-            const int c = ws.counts[bin];
-            clear_mine = !(c > 0 && c <= ch);                 // exactly one work item: it stores this row
-          }
-          break;
-        }
-      }
-    }
-    clear_rows_of_wave(grad_value, i0, value_row_bytes, clear_mine, lane);
-    if (grad_dist != nullptr) clear_rows_of_wave(grad_dist, i0, dist_row_bytes, clear_mine, lane);
-  }
-}
-
 // dst[r, :] = sum over heads m of src[r, m, :], rows of D floats, heads in order; dst is float, or bfloat16
 // when dst16 is set (then D is a multiple of 4)
 __global__ __launch_bounds__(256) void head_sum_kernel(const float *__restrict__ src, void *__restrict__ dst,
@@ -1539,7 +1552,18 @@ static hipError_t run_binning(const BwdArgs &a, const BinWorkspace &ws, int ty, 
   if (LP <= kStage)                         // steps aside if there turn out to be too many bins, as the one above does if not
     hipLaunchKernelGGL(bin_count_kernel, dim3((unsigned)blocks2), dim3(kFillThreads), 0, stream, ws, (const float *)a.loc,
                        a.loc_stride, a.B, a.M, a.L, a.Q, a.P, nq_block, q_blocks2);
-  hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(1024), 0, stream, ws);
+  ClearArgs ca{};
+  unsigned clear_blocks = 0;
+  if (a.clear_grads) {                                   // launch_backward_binned has checked that this applies
+    const int ge = a.grad_bf16 ? 2 : 4;
+    ca.grad_value = static_cast<char *>(a.grad_value);
+    ca.grad_dist = shared_dist(a) ? nullptr : static_cast<char *>(a.grad_dist);   // shared: written whole by the head sum
+    ca.value_row_bytes = a.C * ge; ca.dist_row_bytes = a.D * ge;
+    ca.B = a.B; ca.S = a.S; ca.M = a.M; ca.L = a.L; ca.stores = ((a.C | a.D) & 3) == 0 ? 1 : 0;
+    const size_t rows = (size_t)a.B * a.S * a.M;
+    clear_blocks = (unsigned)((rows + 1023) / 1024 < 4096 ? (rows + 1023) / 1024 : 4096);
+  }
+  hipLaunchKernelGGL(bin_scan_kernel, dim3(1 + clear_blocks), dim3(1024), 0, stream, ws, ca);
   if (LP <= kStage) {
     if (hipError_t e = allow_lds(bin_fill_sorted_kernel, kSortedFillLds)) return e;
     hipLaunchKernelGGL(bin_fill_sorted_kernel, dim3((unsigned)blocks2), dim3(kFillThreads), kSortedFillLds, stream, ws, (const float *)a.loc,
@@ -1566,7 +1590,7 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
     return hipErrorNotSupported;
   if (a.clear_grads) {
     if (kind != 0) return hipErrorInvalidValue;            // the fused entry points only
-    // clear_unstored_kernel writes 16-byte groups where a row is made of them: buffers on 16-byte boundaries,
+    // clear_unstored writes 16-byte groups where a row is made of them: buffers on 16-byte boundaries,
     // or the direct kernels (which clear everything) take the call
     if ((((uintptr_t)a.grad_value | (uintptr_t)a.grad_dist) & 15) != 0) return hipErrorNotSupported;
   }
@@ -1576,14 +1600,6 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
   float *gd_heads = shared_dist(a) ? reinterpret_cast<float *>(static_cast<char *>(workspace) + lay.gd_heads) : nullptr;
   if (a.stage == 0 || a.stage == 1) {
     if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, stream)) return e;
-  }
-  if (a.clear_grads) {
-    const int ge = a.grad_bf16 ? 2 : 4;
-    const size_t rows = (size_t)a.B * a.S * a.M;
-    const unsigned grid = (unsigned)((rows + 255) / 256 < 16384 ? (rows + 255) / 256 : 16384);
-    hipLaunchKernelGGL(clear_unstored_kernel, dim3(grid), dim3(256), 0, stream, ws, static_cast<char *>(a.grad_value),
-                       a.C * ge, gd_heads != nullptr ? nullptr : static_cast<char *>(a.grad_dist), a.D * ge, a.B, a.S, a.M,
-                       a.L, ((a.C | a.D) & 3) == 0 ? 1 : 0);
   }
   if (a.event_binned != nullptr) {
     if (hipError_t e = hipEventRecord((hipEvent_t)a.event_binned, stream)) return e;

@@ -214,7 +214,7 @@ def micro(sections="all"):
 # ------------------------------------------------------------------------------------------------
 KERNEL_KEYS = (("fwd_attention_kernel", "forward"), ("tile_backward_kernel", "backward_tile"),
                ("bin_fill_sorted_kernel", "bin_fill"), ("bin_count_kernel", "bin_count"),
-               ("clear_unstored_kernel", "clear"))
+               ("bin_scan_kernel", "bin_scan_and_clear"))
 
 
 def short_name(n):
@@ -634,7 +634,7 @@ def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
         bin_ms, tile_ms = sum(bin_t) / len(bin_t), sum(tile_t) / len(tile_t)
         kernels["backward_tile"] = entry("tile_backward_kernel (all gradients, one launch)", tile_ms, min(tile_t), bwd_bytes,
                                          "backward_tile")
-        kernels["backward_binning"] = {"kernel": "plan_and_clear + bin_count + bin_scan + bin_fill_sorted (+ their plain forms, which step aside) + clear_unstored",
+        kernels["backward_binning"] = {"kernel": "plan_and_clear + bin_count + bin_scan (whose further blocks clear gradient rows) + bin_fill_sorted (+ their plain forms, which step aside)",
                                        "avg_ms": round(bin_ms, 4), "min_ms": round(min(bin_t), 4)}
         dom = "backward_tile" if tile_ms >= fwd_ms else "forward"
     else:
