@@ -48,8 +48,8 @@ int check_opts(const char *fn, const dfa3d_launch_options *o, dfa3d_launch_optio
     return fail(DFA3D_EINVAL, "%s: options.chunk must be 0 or in [64, 2^20]", fn);
   if (r.clear != 0 && r.clear != 1) return fail(DFA3D_EINVAL, "%s: options.clear must be 0 or 1", fn);
   if (r.clear != 0 && !clear_ok)
-    return fail(DFA3D_EINVAL, "%s: options.clear is for the dfa3d_fused_backward calls only: this call's gradient "
-                "buffers must be zero on entry", fn);
+    return fail(DFA3D_EINVAL, "%s: options.clear is for dfa3d_fused_backward, dfa3d_fused_backward_static and "
+                "dfa3d_wms_deform_attn_backward: this call's gradient buffers must be zero on entry", fn);
   *out = r;
   return 0;
 }
@@ -192,7 +192,7 @@ size_t dfa3d_wms_deform_attn_backward_workspace_bytes(int B, int S, int M, int C
                                                       const dfa3d_launch_options *opts) {
   const char *fn = "dfa3d_wms_deform_attn_backward_workspace_bytes";
   dfa3d_launch_options o;
-  if (check_dims(fn, B, S, M, C, L, Q, P, dtype) || check_opts(fn, opts, &o)) return 0;
+  if (check_dims(fn, B, S, M, C, L, Q, P, dtype) || check_opts(fn, opts, &o, true)) return 0;
   if (o.direct) return 0;
   const dfa3d::BwdArgs a = wms_bwd_args(nullptr, nullptr, 2, nullptr, nullptr, 2, nullptr, nullptr, nullptr, nullptr,
                                         nullptr, 2, nullptr, nullptr, B, S, M, C, L, Q, P, o);
@@ -208,7 +208,7 @@ int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int
   const char *fn = "dfa3d_wms_deform_attn_backward";
   dfa3d_launch_options o;
   if (int rc = check_dims(fn, B, S, M, C, L, Q, P, dtype)) return rc;
-  if (int rc = check_opts(fn, opts, &o)) return rc;
+  if (int rc = check_opts(fn, opts, &o, true)) return rc;
   if (shape_stride < 2 || shape_stride > 3 || loc_stride < 2 || loc_stride > 3 || grad_loc_stride < 2 ||
       grad_loc_stride > 3)
     return fail(DFA3D_EINVAL, "%s: shape_stride, loc_stride and grad_loc_stride must be 2 or 3", fn);
@@ -222,6 +222,11 @@ int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int
   if (workspace != nullptr && !o.direct) {
     const hipError_t e = dfa3d::launch_backward_binned(a, dtype, workspace, workspace_bytes, (hipStream_t)stream);
     if (e != hipErrorNotSupported) return hip_result(e, fn);
+  }
+  if (a.clear_grads) {          // the direct kernels add every term into grad_value: all of it is cleared first
+    if (hipError_t e = dfa3d::launch_zero_fill(grad_value, (size_t)B * S * M * C * (dtype == DFA3D_F64 ? 8 : 4),
+                                               (hipStream_t)stream))
+      return hip_result(e, fn);
   }
   return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
 }

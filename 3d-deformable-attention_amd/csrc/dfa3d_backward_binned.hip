@@ -1557,9 +1557,11 @@ static hipError_t run_binning(const BwdArgs &a, const BinWorkspace &ws, int ty, 
   if (a.clear_grads) {                                   // launch_backward_binned has checked that this applies
     const int ge = a.grad_bf16 ? 2 : 4;
     ca.grad_value = static_cast<char *>(a.grad_value);
-    ca.grad_dist = shared_dist(a) ? nullptr : static_cast<char *>(a.grad_dist);   // shared: written whole by the head sum
+    // no grad_dist in stage 2 alone; for a distribution shared by the heads the head sum writes all of it
+    ca.grad_dist = (a.dist == nullptr || shared_dist(a)) ? nullptr : static_cast<char *>(a.grad_dist);
     ca.value_row_bytes = a.C * ge; ca.dist_row_bytes = a.D * ge;
-    ca.B = a.B; ca.S = a.S; ca.M = a.M; ca.L = a.L; ca.stores = ((a.C | a.D) & 3) == 0 ? 1 : 0;
+    ca.B = a.B; ca.S = a.S; ca.M = a.M; ca.L = a.L;
+    ca.stores = ((a.C | (a.dist != nullptr ? a.D : 0)) & 3) == 0 ? 1 : 0;        // the tile kernel's own condition
     const size_t rows = (size_t)a.B * a.S * a.M;
     clear_blocks = (unsigned)((rows + 1023) / 1024 < 4096 ? (rows + 1023) / 1024 : 4096);
   }
@@ -1589,7 +1591,7 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
   if (need == 0 || workspace == nullptr || workspace_bytes < need || ((uintptr_t)workspace & 255) != 0)
     return hipErrorNotSupported;
   if (a.clear_grads) {
-    if (kind != 0) return hipErrorInvalidValue;            // the fused entry points only
+    if (kind == 2) return hipErrorInvalidValue;            // the depth-only tile kernel stores nothing
     // clear_unstored writes 16-byte groups where a row is made of them: buffers on 16-byte boundaries,
     // or the direct kernels (which clear everything) take the call
     if ((((uintptr_t)a.grad_value | (uintptr_t)a.grad_dist) & 15) != 0) return hipErrorNotSupported;

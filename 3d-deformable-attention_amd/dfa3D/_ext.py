@@ -184,7 +184,18 @@ def wms_deform_attn_backward(value, value_spatial_shapes, value_level_start_inde
                              attention_weights, depth_scores, grad_output, grad_value, grad_sampling_loc,
                              grad_attn_weight, grad_depth_score, im2col_step):
     """Accumulates into ``grad_value`` (pre-zeroed by the caller); overwrites the x, y components of
-    ``grad_sampling_loc``, ``grad_attn_weight`` and ``grad_depth_score``."""
+    ``grad_sampling_loc``, ``grad_attn_weight`` and ``grad_depth_score``.  Names and order of the arguments are the
+    reference's (pybind.cpp:48-54)."""
+    wms_deform_attn_backward_into(value, value_spatial_shapes, value_level_start_index, sampling_locations,
+                                  attention_weights, depth_scores, grad_output, grad_value, grad_sampling_loc,
+                                  grad_attn_weight, grad_depth_score, im2col_step, clear=False)
+
+
+def wms_deform_attn_backward_into(value, value_spatial_shapes, value_level_start_index, sampling_locations,
+                                  attention_weights, depth_scores, grad_output, grad_value, grad_sampling_loc,
+                                  grad_attn_weight, grad_depth_score, im2col_step, clear=False):
+    """``wms_deform_attn_backward`` with one more choice: ``clear=True`` takes a ``grad_value`` that holds anything
+    (``torch.empty``) and clears what the kernels add to rather than store (see ``dfa3d_fused_backward``)."""
     _contig(value=value, spatial_shapes=value_spatial_shapes, level_start_index=value_level_start_index,
             sampling_loc=sampling_locations, attn_weight=attention_weights, depth_score=depth_scores,
             grad_output=grad_output, grad_value=grad_value, grad_sampling_loc=grad_sampling_loc,
@@ -208,17 +219,20 @@ def wms_deform_attn_backward(value, value_spatial_shapes, value_level_start_inde
     _expect(grad_depth_score, "grad_depth_score", shape=(B, Q, M, L, P, 4), dtype=aux)
     _step(B, im2col_step)
     if grad_output.numel() == 0:
+        if clear:
+            grad_value.zero_()
         return
     code = _lib.dtype_code(value)
-    ws_bytes = _lib.lib().dfa3d_wms_deform_attn_backward_workspace_bytes(B, S, M, C, L, Q, P, code, _lib.options())
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
-    with torch.cuda.device(dev):
-        rc = _lib.lib().dfa3d_wms_deform_attn_backward(
-            _lib.ptr(value), _lib.ptr(value_spatial_shapes), sw, _lib.ptr(value_level_start_index),
-            _lib.ptr(sampling_locations), lw, _lib.ptr(attention_weights), _lib.ptr(depth_scores),
-            _lib.ptr(grad_output), _lib.ptr(grad_value), _lib.ptr(grad_sampling_loc), gw, _lib.ptr(grad_attn_weight),
-            _lib.ptr(grad_depth_score), _lib.ptr(workspace), ws_bytes, B, S, M, C, L, Q, P, code, _lib.options(),
-            _lib.stream_of(value))
+    with (_lib.launch_options(clear=1) if clear else contextlib.nullcontext()):
+        ws_bytes = _lib.lib().dfa3d_wms_deform_attn_backward_workspace_bytes(B, S, M, C, L, Q, P, code, _lib.options())
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
+        with torch.cuda.device(dev):
+            rc = _lib.lib().dfa3d_wms_deform_attn_backward(
+                _lib.ptr(value), _lib.ptr(value_spatial_shapes), sw, _lib.ptr(value_level_start_index),
+                _lib.ptr(sampling_locations), lw, _lib.ptr(attention_weights), _lib.ptr(depth_scores),
+                _lib.ptr(grad_output), _lib.ptr(grad_value), _lib.ptr(grad_sampling_loc), gw,
+                _lib.ptr(grad_attn_weight), _lib.ptr(grad_depth_score), _lib.ptr(workspace), ws_bytes, B, S, M, C, L,
+                Q, P, code, _lib.options(), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_wms_deform_attn_backward")
 
 
@@ -249,9 +263,10 @@ def ms_deform_attn_forward(value, value_spatial_shapes, value_level_start_index,
 
 def ms_deform_attn_backward(value, value_spatial_shapes, value_level_start_index, sampling_locations,
                             attention_weights, grad_output, grad_value, grad_sampling_loc, grad_attn_weight,
-                            im2col_step):
+                            im2col_step, clear=False):
     """Backward of ms_deform_attn_forward (…/multi_scale_deformable_attn_function.py:74-84).  Accumulates into
-    ``grad_value`` (pre-zeroed by the caller); overwrites ``grad_sampling_loc`` and ``grad_attn_weight``."""
+    ``grad_value`` (pre-zeroed by the caller, or holding anything with ``clear=True``); overwrites
+    ``grad_sampling_loc`` and ``grad_attn_weight``."""
     named = dict(value=value, spatial_shapes=value_spatial_shapes, level_start_index=value_level_start_index,
                  sampling_loc=sampling_locations, attn_weight=attention_weights, grad_output=grad_output,
                  grad_value=grad_value, grad_sampling_loc=grad_sampling_loc, grad_attn_weight=grad_attn_weight)
@@ -268,16 +283,19 @@ def ms_deform_attn_backward(value, value_spatial_shapes, value_level_start_index
     _expect(grad_attn_weight, "grad_attn_weight", shape=(B, Q, M, L, P), dtype=aux)
     _step(B, im2col_step)
     if grad_output.numel() == 0:
+        if clear:
+            grad_value.zero_()
         return
     code = _lib.dtype_code(value)
-    ws_bytes = _lib.lib().dfa3d_wms_deform_attn_backward_workspace_bytes(B, S, M, C, L, Q, P, code, _lib.options())
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
-    with torch.cuda.device(dev):
-        rc = _lib.lib().dfa3d_wms_deform_attn_backward(
-            _lib.ptr(value), _lib.ptr(value_spatial_shapes), sw, _lib.ptr(value_level_start_index),
-            _lib.ptr(sampling_locations), lw, _lib.ptr(attention_weights), None, _lib.ptr(grad_output),
-            _lib.ptr(grad_value), _lib.ptr(grad_sampling_loc), lw, _lib.ptr(grad_attn_weight), None,
-            _lib.ptr(workspace), ws_bytes, B, S, M, C, L, Q, P, code, _lib.options(), _lib.stream_of(value))
+    with (_lib.launch_options(clear=1) if clear else contextlib.nullcontext()):
+        ws_bytes = _lib.lib().dfa3d_wms_deform_attn_backward_workspace_bytes(B, S, M, C, L, Q, P, code, _lib.options())
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
+        with torch.cuda.device(dev):
+            rc = _lib.lib().dfa3d_wms_deform_attn_backward(
+                _lib.ptr(value), _lib.ptr(value_spatial_shapes), sw, _lib.ptr(value_level_start_index),
+                _lib.ptr(sampling_locations), lw, _lib.ptr(attention_weights), None, _lib.ptr(grad_output),
+                _lib.ptr(grad_value), _lib.ptr(grad_sampling_loc), lw, _lib.ptr(grad_attn_weight), None,
+                _lib.ptr(workspace), ws_bytes, B, S, M, C, L, Q, P, code, _lib.options(), _lib.stream_of(value))
     _lib.check(rc, "dfa3d_wms_deform_attn_backward")
 
 

@@ -110,16 +110,16 @@ class WeightedMultiScaleDeformableAttnFunction(Function):
         value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights, \
             depth_score = ctx.saved_tensors
         aux = _aux(value)
-        grad_value = torch.zeros(value.shape, dtype=aux, device=value.device)
+        grad_value = torch.empty(value.shape, dtype=aux, device=value.device)      # cleared by the call (clear=True)
         grad_sampling_loc = torch.empty_like(sampling_locations)
         if sampling_locations.shape[-1] > 2:
             grad_sampling_loc[..., 2:] = 0
         grad_attn_weight = torch.empty_like(attention_weights)
         grad_depth_score = torch.empty(depth_score.shape, dtype=aux, device=value.device)
-        _ext.wms_deform_attn_backward(
+        _ext.wms_deform_attn_backward_into(
             value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights,
             depth_score, _grad_in(grad_output, value.dtype), grad_value, grad_sampling_loc, grad_attn_weight,
-            grad_depth_score, im2col_step=ctx.im2col_step)
+            grad_depth_score, im2col_step=ctx.im2col_step, clear=True)
         return grad_value.to(value.dtype), None, None, grad_sampling_loc, grad_attn_weight, \
             grad_depth_score.to(depth_score.dtype), None
 
@@ -144,7 +144,7 @@ class MultiScaleDeformableAttnFunction(Function):
     def backward(ctx, grad_output):
         value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights = \
             ctx.saved_tensors
-        grad_value = torch.zeros(value.shape, dtype=_aux(value), device=value.device)
+        grad_value = torch.empty(value.shape, dtype=_aux(value), device=value.device)   # cleared by the call
         grad_sampling_loc = torch.empty_like(sampling_locations)
         if sampling_locations.shape[-1] > 2:
             grad_sampling_loc[..., 2:] = 0
@@ -152,7 +152,7 @@ class MultiScaleDeformableAttnFunction(Function):
         _ext.ms_deform_attn_backward(
             value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights,
             _grad_in(grad_output, value.dtype), grad_value, grad_sampling_loc, grad_attn_weight,
-            im2col_step=ctx.im2col_step)
+            im2col_step=ctx.im2col_step, clear=True)
         return grad_value.to(value.dtype), None, None, grad_sampling_loc, grad_attn_weight, None
 
 

@@ -63,10 +63,10 @@ typedef struct dfa3d_launch_options {
   int block;    /* binned backward: threads per tile workgroup, 256 or 0/512 */
   int pass;     /* binned backward: points a tile workgroup takes per pass, 64, 128 or 256; 0 = automatic */
   int chunk;    /* binned backward: points of one tile handled by one work item, 0 = 4096 */
-  int clear;    /* dfa3d_fused_backward / dfa3d_fused_backward_static only (0 elsewhere): non-zero = grad_value and
-                 * grad_dist may hold anything on entry, the call clears what its kernels add to instead of
-                 * storing (a quarter of the buffers with the tile kernel, all of them otherwise); 0 = they are
-                 * zero on entry, as the reference's caller makes them */
+  int clear;    /* dfa3d_fused_backward, dfa3d_fused_backward_static and dfa3d_wms_deform_attn_backward only (0
+                 * elsewhere): non-zero = grad_value (and grad_dist) may hold anything on entry, the call clears what
+                 * its kernels add to instead of storing (a quarter of the buffers with the tile kernel, all of
+                 * them otherwise); 0 = they are zero on entry, as the reference's caller makes them */
   void *event_binned;   /* a hipEvent_t, or NULL: a binned backward records it on `stream` between its binning
                          * kernels and its tile kernel, so that a profiler can time the two parts of the call */
 } dfa3d_launch_options;
@@ -110,7 +110,7 @@ int dfa3d_wms_deform_attn_forward(
     void *out,
     int B, int S, int M, int C, int L, int Q, int P, int dtype, const dfa3d_launch_options *opts, void *stream);
 
-/* Stage 2 backward.  `grad_value` must be zero on entry and holds the gradient on return;
+/* Stage 2 backward.  `grad_value` must be zero on entry (or options.clear is set) and holds the gradient on return;
  * `grad_loc` (B,Q,M,L,P,grad_loc_stride) gets its first two components overwritten, `grad_attn` and
  * `grad_score` are overwritten (`score` == NULL: scores all 1, `grad_score` may be NULL and is then not
  * written).  `workspace` as for dfa3d_fused_backward (size from

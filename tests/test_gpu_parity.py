@@ -572,6 +572,38 @@ def test_gradient_buffers_that_were_not_zeroed(variant):
     assert want_gv.abs().sum() > 0 and want_gd.abs().sum() > 0
 
 
+@pytest.mark.parametrize("variant", ["scores", "plain", "plain-direct", "odd-channels"])
+def test_stage_two_gradient_buffer_that_was_not_zeroed(variant):
+    """options.clear on the stage-2 backward (depth scores given, or none: plain deformable attention): a grad_value
+    full of NaN comes back equal to what the call writes into a zeroed one."""
+    from dfa3D import _ext, _lib
+    dev = _dev()
+    kw = dict(seed=310, B=2, M=8, C=32, D=4, Q=400, P=4, levels=((37, 52), (19, 26), (5, 3)), dtype=torch.float32)
+    if variant == "odd-channels":
+        kw.update(C=6)
+    t = tiny_case(**kw)
+    t["loc"][:, :, :, 0] = t["loc"][:, :, :, 0] * 0.3            # level 0: most tiles stay without points
+    value, loc, attn, go = [t[k].to(dev) for k in ("value", "loc", "attn", "grad_out")]
+    shapes3, lsi = t["shapes3"].to(dev), t["lsi"].to(dev)
+    score = torch.rand(*attn.shape, 4, device=dev)
+    opts = dict(direct=1) if variant == "plain-direct" else {}
+
+    def run(fill, clear):
+        gv = torch.full(value.shape, fill, device=dev)
+        gl, ga, gs = torch.zeros_like(loc), torch.empty_like(attn), torch.empty_like(score)
+        with _lib.launch_options(**opts):
+            if variant.startswith("plain"):
+                _ext.ms_deform_attn_backward(value, shapes3, lsi, loc, attn, go, gv, gl, ga, 64, clear=clear)
+            else:
+                _ext.wms_deform_attn_backward_into(value, shapes3, lsi, loc, attn, score, go, gv, gl, ga, gs, 64, clear=clear)
+        torch.cuda.synchronize()
+        return gv.cpu()
+
+    want, got = run(0.0, False), run(float("nan"), True)
+    assert torch.isfinite(got).all() and want.abs().sum() > 0
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
+
+
 def _random_case_with_options(seed):
     """A wider draw than _random_case (channel counts up to 256, depth bins up to 128, up to 3000 queries on maps of
     1 to 60 pixels a side, locations inside, around and in a corner of the map) with launch options drawn from
