@@ -41,7 +41,7 @@ namespace dfa3d {
 constexpr int kClasses = 8;         // work queues: one per XCD (workgroup id % 8 with round-robin placement)
 constexpr int kQueueStride = 16;    // ints between queue counters: one 64-byte line each
 constexpr int kQueueInts = kClasses * kQueueStride + 32;   // + room for the optional phase timers
-constexpr int kBinQueries = 32;     // queries of one (batch, head) handled by a count/fill block (16, 64, 128 time worse)
+constexpr int kBinQueries = 32;     // bin_points_kernel: queries of one (batch, head) per block step (16, 64, 128 time worse)
 constexpr int kHistCap = 8192;      // bins of one (batch, head) that fit the LDS histogram
 
 struct BinPlan {
@@ -426,7 +426,7 @@ __device__ __forceinline__ void clear_rows_of_wave(char *base, size_t first_row,
 }
 
 struct ClearArgs {
-  char *grad_value, *grad_dist;     // grad_value == nullptr: nothing to clear; grad_dist == nullptr: not that one
+  char *grad_value, *grad_dist;     // either may be nullptr: not that one
   int value_row_bytes, dist_row_bytes, B, S, M, L, stores;
 };
 __device__ __forceinline__ void clear_unstored(const BinWorkspace &ws, const ClearArgs &ca, unsigned block, unsigned n_blocks) {
@@ -458,7 +458,7 @@ __device__ __forceinline__ void clear_unstored(const BinWorkspace &ws, const Cle
         }
       }
     }
-    clear_rows_of_wave(grad_value, i0, value_row_bytes, clear_mine, lane);
+    if (grad_value != nullptr) clear_rows_of_wave(grad_value, i0, value_row_bytes, clear_mine, lane);
     if (grad_dist != nullptr) clear_rows_of_wave(grad_dist, i0, dist_row_bytes, clear_mine, lane);
   }
 }
@@ -1531,7 +1531,7 @@ static BinWorkspace carve_workspace(void *workspace, const BinLayout &lay) {
 
 // plan, count, scan, fill.  `a` supplies dimensions, shapes, locations and the per-point gradient
 // buffers that receive zeros for points the operator skips.
-static hipError_t run_binning(const BwdArgs &a, const BinWorkspace &ws, int ty, int tx, hipStream_t stream) {
+static hipError_t run_binning(const BwdArgs &a, const BinWorkspace &ws, int ty, int tx, float *gd_heads, hipStream_t stream) {
   const int mb = max_bins_per_bm(a.S, a.L, ty, tx);
   hipLaunchKernelGGL(plan_and_clear_kernel, dim3(64), dim3(256), 0, stream, ws, a.shapes, a.shape_stride, a.level_start,
                      a.L, a.S, (a.dist != nullptr || a.C == 0) ? a.D : 0, a.B, a.M, ty, tx, a.chunk_hint > 0 ? a.chunk_hint : kDefaultChunk, mb);
@@ -1552,14 +1552,18 @@ static hipError_t run_binning(const BwdArgs &a, const BinWorkspace &ws, int ty, 
   if (LP <= kStage)                         // steps aside if there turn out to be too many bins, as the one above does if not
     hipLaunchKernelGGL(bin_count_kernel, dim3((unsigned)blocks2), dim3(kFillThreads), 0, stream, ws, (const float *)a.loc,
                        a.loc_stride, a.B, a.M, a.L, a.Q, a.P, nq_block, q_blocks2);
+  // What further blocks of the scan's launch clear meanwhile: for a caller that did not zero them (options.clear),
+  // the rows of grad_value / grad_dist that the tile kernel adds to rather than stores; and always, for a
+  // distribution shared by the heads, those rows of the per-head grad_dist in the workspace (the head sum then
+  // writes all of the caller's grad_dist).
   ClearArgs ca{};
   unsigned clear_blocks = 0;
-  if (a.clear_grads) {                                   // launch_backward_binned has checked that this applies
+  if (a.clear_grads || gd_heads != nullptr) {            // launch_backward_binned has checked that this applies
     const int ge = a.grad_bf16 ? 2 : 4;
-    ca.grad_value = static_cast<char *>(a.grad_value);
-    // no grad_dist in stage 2 alone; for a distribution shared by the heads the head sum writes all of it
-    ca.grad_dist = (a.dist == nullptr || shared_dist(a)) ? nullptr : static_cast<char *>(a.grad_dist);
-    ca.value_row_bytes = a.C * ge; ca.dist_row_bytes = a.D * ge;
+    ca.grad_value = a.clear_grads ? static_cast<char *>(a.grad_value) : nullptr;
+    ca.value_row_bytes = a.C * ge;
+    if (gd_heads != nullptr) { ca.grad_dist = reinterpret_cast<char *>(gd_heads); ca.dist_row_bytes = a.D * 4; }
+    else if (a.dist != nullptr) { ca.grad_dist = static_cast<char *>(a.grad_dist); ca.dist_row_bytes = a.D * ge; }
     ca.B = a.B; ca.S = a.S; ca.M = a.M; ca.L = a.L;
     ca.stores = ((a.C | (a.dist != nullptr ? a.D : 0)) & 3) == 0 ? 1 : 0;        // the tile kernel's own condition
     const size_t rows = (size_t)a.B * a.S * a.M;
@@ -1601,14 +1605,14 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
   const BinWorkspace ws = carve_workspace(workspace, lay);
   float *gd_heads = shared_dist(a) ? reinterpret_cast<float *>(static_cast<char *>(workspace) + lay.gd_heads) : nullptr;
   if (a.stage == 0 || a.stage == 1) {
-    if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, stream)) return e;
+    if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, gd_heads, stream)) return e;
   }
   if (a.event_binned != nullptr) {
     if (hipError_t e = hipEventRecord((hipEvent_t)a.event_binned, stream)) return e;
   }
   if (a.stage == 1) return hipSuccess;
   const size_t head_floats = (size_t)a.B * a.S * a.M * a.D;
-  if (gd_heads != nullptr)       // a kernel, not a memset node: callers may capture this stream in a graph
+  if (gd_heads != nullptr && a.stage == 2)       // (development builds: tile kernel without the binning launches)
     hipLaunchKernelGGL(fill_zero_kernel, dim3(2048), dim3(256), 0, stream, reinterpret_cast<float4 *>(gd_heads),
                        (head_floats + 3) / 4);
   if (a.grad_bf16 && dtype != DFA3D_BF16) return hipErrorInvalidValue;
@@ -1641,7 +1645,7 @@ hipError_t launch_depth_score_backward_binned(const DepthScoreBwdArgs &d, int dt
     return hipErrorNotSupported;
   const TileConfig cfg = tile_config_of(a, 2);
   const BinWorkspace ws = carve_workspace(workspace, bin_layout(a, cfg.ty, cfg.tx));
-  if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, stream)) return e;
+  if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, nullptr, stream)) return e;
   if (event_binned != nullptr) {
     if (hipError_t e = hipEventRecord((hipEvent_t)event_binned, stream)) return e;
   }
