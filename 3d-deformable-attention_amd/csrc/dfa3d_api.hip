@@ -67,8 +67,6 @@ void apply_opts(dfa3d::BwdArgs &a, const dfa3d_launch_options &o) {
 #ifdef DFA3D_EXPERIMENT
   a.diag = g_diag.load(std::memory_order_relaxed);
   a.stage = g_stage.load(std::memory_order_relaxed);
-#else
-  a.diag = 0; a.stage = 0;
 #endif
 }
 
@@ -108,6 +106,7 @@ int dfa3d_experiment_set(const char *name, int value) {
   if (name != nullptr && !strcmp(name, "bwd_stage")) { g_stage.store(value, std::memory_order_relaxed); return 0; }
   return fail(DFA3D_EINVAL, "dfa3d_experiment_set: unknown switch");
 }
+size_t dfa3d_experiment_timer_offset(void) { return dfa3d::tile_timer_offset(); }
 #endif
 
 int dfa3d_ms_depth_score_sample_forward(const void *dist, const int64_t *shapes3, const int64_t *level_start,
@@ -231,7 +230,8 @@ int dfa3d_wms_deform_attn_backward(const void *value, const int64_t *shapes, int
   return hip_result(dfa3d::launch_backward(a, dtype, (hipStream_t)stream), fn);
 }
 
-// cells of a packed distribution: sum over levels of (H + 1)(W + 1) <= sum of (2 H W + 2) <= 2 S + 2 L
+// cells of a packed distribution: sum over levels of (H + 1)(W + 1) <= sum of (2 H W + 2) <= 2 S + 2 L for levels that
+// share no keys; the kernels check the level table they find on the device against the same bound
 static long long packed_cells_bound(int S, int L) { return 2LL * S + 2LL * L; }
 
 size_t dfa3d_packed_dist_bytes(int B, int S, int D, int L, int dtype) {

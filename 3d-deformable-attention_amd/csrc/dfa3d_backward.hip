@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kBlock) void bwd_attention_kernel(
     const T *__restrict__ grad_score_in, A *__restrict__ grad_value, A *__restrict__ grad_dist,
     A *__restrict__ grad_loc, int gl_stride, A *__restrict__ grad_attn, A *__restrict__ grad_score_out,
     const A *__restrict__ grad_wu, int Md,
-    int B, int S, int M, int C, int D, int L, int Q, int P, int iters, int q_blocks, int diag) {
+    int B, int S, int M, int C, int D, int L, int Q, int P, int iters, int q_blocks DFA3D_DIAG_PARAM) {
   __shared__ LevelTable tab;
   __shared__ Task<A> s_tasks[kWavesPerBlock][kWave * 4];
   __shared__ A s_dots[kWavesPerBlock][kWave * 4];
@@ -347,14 +347,14 @@ static hipError_t launch_bwd_cfg(const BwdArgs &a, hipStream_t stream) {
                        (const T *)a.grad_out, (const T *)a.grad_score_in, (A *)a.grad_value, (A *)a.grad_dist,
                        (A *)a.grad_loc, a.grad_loc_stride, (A *)a.grad_attn, (A *)nullptr,
                        (const A *)a.grad_weight_update, a.dist_heads == 1 ? 1 : a.M, a.B, a.S, a.M, a.C, a.D,
-                       a.L, a.Q, a.P, iters, q_blocks, a.diag);
+                       a.L, a.Q, a.P, iters, q_blocks DFA3D_DIAG_ARG(a));
   } else {
     hipLaunchKernelGGL((bwd_attention_kernel<T, A, VEC, LPR, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,
                        (const T *)a.value, (const T *)nullptr, a.shapes, a.shape_stride, a.level_start,
                        (const A *)a.loc, a.loc_stride, (const A *)a.attn, (const T *)a.score_in,
                        (const T *)a.grad_out, (const T *)nullptr, (A *)a.grad_value, (A *)nullptr, (A *)a.grad_loc,
                        a.grad_loc_stride, (A *)a.grad_attn, (A *)a.grad_score_out, (const A *)nullptr, a.M, a.B, a.S,
-                       a.M, a.C, a.D, a.L, a.Q, a.P, iters, q_blocks, a.diag);
+                       a.M, a.C, a.D, a.L, a.Q, a.P, iters, q_blocks DFA3D_DIAG_ARG(a));
   }
   return hipGetLastError();
 }

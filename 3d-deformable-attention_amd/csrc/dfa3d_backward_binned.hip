@@ -155,7 +155,7 @@ template <int MODE>
 __global__ __launch_bounds__(256) void bin_points_kernel(
     BinWorkspace ws, const float *__restrict__ loc, int loc_stride, const float *__restrict__ attn,
     float *__restrict__ grad_loc, int gl_stride, float *__restrict__ grad_attn, float *__restrict__ grad_score,
-    int B, int M, int L, int Q, int P, int q_blocks, int n_blocks, int hist_cap, int diag) {
+    int B, int M, int L, int Q, int P, int q_blocks, int n_blocks, int hist_cap DFA3D_DIAG_PARAM) {
   extern __shared__ int s_hist[];          // [0, nb): counts, then for MODE 1 [nb, 2 nb): segment bases
   const BinPlan &p = *ws.plan;
   const int nb = p.bins_per_bm;
@@ -677,7 +677,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
     const T *__restrict__ grad_out, const T *__restrict__ grad_score_in,
     void *__restrict__ grad_value, void *__restrict__ grad_dist, float *__restrict__ grad_loc, int gl_stride,
     float *__restrict__ grad_attn, float *__restrict__ grad_score_out, const float *__restrict__ grad_wu, int Md,
-    int Mg, int B, int S, int M, int C, int D, int L, int Q, int P, int PP, int grad16, int diag) {
+    int Mg, int B, int S, int M, int C, int D, int L, int Q, int P, int PP, int grad16 DFA3D_DIAG_PARAM) {
   // grad16: bit 0 = grad_value is bfloat16, bit 1 = grad_dist is bfloat16 (else float)
   // Md: heads stored in dist (M, or 1 = shared by all heads); Mg: heads of the grad_dist buffer written here
   constexpr int RPI = kWave / LPR;                  // row groups per wavefront
@@ -929,11 +929,15 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         const uint32_t chan_off = chan < C ? (uint32_t)(chan * sizeof(T)) : kNoChan;
 #pragma unroll 4
         for (int j = 0; j < stage_per_wave; j += RPI) {
-          const int slot = wave * stage_per_wave + j + lane / LPR;
+          // a wavefront with fewer rows to stage than row groups (short passes, few lanes per row) leaves the
+          // groups beyond its share idle: their slots belong to the next wavefront, or lie past the last one
+          const int sub = j + lane / LPR;
+          const bool slot_ok = sub < stage_per_wave;
+          const int slot = wave * stage_per_wave + min(sub, stage_per_wave - 1);
           float gg[VEC];
           if (DFA3D_DIAG(diag, 256)) { for (int i = 0; i < VEC; ++i) gg[i] = 1.f; } else   // cost of the grad_out loads
           RowVec<T, float, VEC>::ld(go_r, goff[slot] + chan_off, gg);
-          if (chan < C) LdsVec<VEC>::st(gstage + slot * C + chan, gg);
+          if (slot_ok && chan < C) LdsVec<VEC>::st(gstage + slot * C + chan, gg);
         }
       }
       __syncthreads();                                   // counts complete
@@ -1353,6 +1357,13 @@ static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
   return o;
 }
 
+#ifdef DFA3D_EXPERIMENT
+// development builds: where in a workspace the tile kernel's phase clocks live (ten 64-bit counters)
+size_t tile_timer_offset() {
+  return ((sizeof(BinPlan) + 255) & ~(size_t)255) + (size_t)kClasses * kQueueStride * sizeof(int);
+}
+#endif
+
 // Launch shape of the tile kernels: tile edge, threads per workgroup, points per pass.
 struct TileConfig { int ty, tx, block, pp; size_t lds; };
 
@@ -1484,7 +1495,7 @@ static hipError_t launch_tile_cfg(const BwdArgs &a, const BinWorkspace &ws, cons
                        gd_heads != nullptr ? (void *)gd_heads : a.grad_dist, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
                        (float *)nullptr, (const float *)a.grad_weight_update, a.dist_heads == 1 ? 1 : a.M,
                        (a.dist_heads == 1 && gd_heads == nullptr) ? 1 : a.M, a.B, a.S, a.M, a.C, a.D, a.L, a.Q, a.P, c.pp,
-                       (a.grad_bf16 ? 1 : 0) | ((a.grad_bf16 && gd_heads == nullptr) ? 2 : 0), a.diag);
+                       (a.grad_bf16 ? 1 : 0) | ((a.grad_bf16 && gd_heads == nullptr) ? 2 : 0) DFA3D_DIAG_ARG(a));
   } else {
     auto kern = tile_backward_kernel<T, VEC, LPR, false>;
     if (hipError_t e = allow_lds(kern, c.lds)) return e;
@@ -1492,7 +1503,7 @@ static hipError_t launch_tile_cfg(const BwdArgs &a, const BinWorkspace &ws, cons
                        (const T *)a.score_in, (const T *)a.grad_out, (const T *)nullptr, a.grad_value,
                        (void *)nullptr, (float *)a.grad_loc, a.grad_loc_stride, (float *)a.grad_attn,
                        (float *)a.grad_score_out, (const float *)nullptr, a.M, a.M, a.B, a.S, a.M, a.C, 0, a.L, a.Q,
-                       a.P, c.pp, 0, a.diag);
+                       a.P, c.pp, 0 DFA3D_DIAG_ARG(a));
   }
   return hipGetLastError();
 }
@@ -1542,8 +1553,7 @@ static hipError_t run_binning(const BwdArgs &a, const BinWorkspace &ws, int ty, 
   const unsigned grid = blocks < 2048 ? (unsigned)blocks : 2048u;
   hipLaunchKernelGGL(bin_points_kernel<0>, dim3(grid), dim3(256), (size_t)hist_cap * 4, stream, ws,
                      (const float *)a.loc, a.loc_stride, (const float *)a.attn, (float *)a.grad_loc, a.grad_loc_stride,
-                     (float *)a.grad_attn, (float *)a.grad_score_out, a.B, a.M, a.L, a.Q, a.P, q_blocks, (int)blocks, hist_cap,
-                     a.diag);
+                     (float *)a.grad_attn, (float *)a.grad_score_out, a.B, a.M, a.L, a.Q, a.P, q_blocks, (int)blocks, hist_cap DFA3D_DIAG_ARG(a));
   const int LP = a.L * a.P;
   const int nq_block = LP <= kStage ? kStage / LP : 1;
   const int q_blocks2 = (a.Q + nq_block - 1) / nq_block;
@@ -1578,8 +1588,7 @@ static hipError_t run_binning(const BwdArgs &a, const BinWorkspace &ws, int ty, 
   }
   hipLaunchKernelGGL(bin_points_kernel<1>, dim3(grid), dim3(256), (size_t)hist_cap * 8, stream, ws,
                      (const float *)a.loc, a.loc_stride, (const float *)a.attn, (float *)a.grad_loc, a.grad_loc_stride,
-                     (float *)a.grad_attn, (float *)a.grad_score_out, a.B, a.M, a.L, a.Q, a.P, q_blocks, (int)blocks, hist_cap,
-                     a.diag);
+                     (float *)a.grad_attn, (float *)a.grad_score_out, a.B, a.M, a.L, a.Q, a.P, q_blocks, (int)blocks, hist_cap DFA3D_DIAG_ARG(a));
   return hipGetLastError();
 }
 
@@ -1604,17 +1613,21 @@ hipError_t launch_backward_binned(const BwdArgs &a, int dtype, void *workspace, 
   const BinLayout lay = bin_layout(a, cfg.ty, cfg.tx);
   const BinWorkspace ws = carve_workspace(workspace, lay);
   float *gd_heads = shared_dist(a) ? reinterpret_cast<float *>(static_cast<char *>(workspace) + lay.gd_heads) : nullptr;
-  if (a.stage == 0 || a.stage == 1) {
+#ifdef DFA3D_EXPERIMENT
+  const int stage = a.stage;                     // development builds: 1 = binning launches only, 2 = tile kernel only
+#else
+  constexpr int stage = 0;
+#endif
+  if (stage == 0 || stage == 1) {
     if (hipError_t e = run_binning(a, ws, cfg.ty, cfg.tx, gd_heads, stream)) return e;
   }
   if (a.event_binned != nullptr) {
     if (hipError_t e = hipEventRecord((hipEvent_t)a.event_binned, stream)) return e;
   }
-  if (a.stage == 1) return hipSuccess;
-  const size_t head_floats = (size_t)a.B * a.S * a.M * a.D;
-  if (gd_heads != nullptr && a.stage == 2)       // (development builds: tile kernel without the binning launches)
+  if (stage == 1) return hipSuccess;
+  if (gd_heads != nullptr && stage == 2)
     hipLaunchKernelGGL(fill_zero_kernel, dim3(2048), dim3(256), 0, stream, reinterpret_cast<float4 *>(gd_heads),
-                       (head_floats + 3) / 4);
+                       ((size_t)a.B * a.S * a.M * a.D + 3) / 4);
   if (a.grad_bf16 && dtype != DFA3D_BF16) return hipErrorInvalidValue;
   const hipError_t e = dtype == DFA3D_F32 ? launch_tile_typed<float>(a, ws, cfg, gd_heads, stream)
                                           : launch_tile_typed<__hip_bfloat16>(a, ws, cfg, gd_heads, stream);

@@ -28,8 +28,12 @@ namespace dfa3d {
 // in the library as shipped the switches are constant zero and the compiler drops them.
 #ifdef DFA3D_EXPERIMENT
 #define DFA3D_DIAG(diag, bits) (((diag) & (bits)) != 0)
+#define DFA3D_DIAG_PARAM , int diag          // last kernel parameter, development builds only
+#define DFA3D_DIAG_ARG(a) , (a).diag
 #else
 #define DFA3D_DIAG(diag, bits) false
+#define DFA3D_DIAG_PARAM
+#define DFA3D_DIAG_ARG(a)
 #endif
 
 constexpr int kWave = 64;
@@ -274,6 +278,9 @@ __device__ __forceinline__ void load_cell_starts(LevelTable &tab, int L) {
   }
   __syncthreads();
 }
+
+// Cells the host sizes a packed table for: levels that share no keys have sum (H + 1)(W + 1) <= 2 S + 2 L of them.
+__host__ __device__ inline long long packed_cell_capacity(int S, int L) { return 2LL * S + 2LL * L; }
 
 // bins (d, d + 1) of one cell: 8 elements, 32 bytes (16 for bfloat16), one cache line access
 template <typename T> struct PackedTap;

@@ -56,14 +56,18 @@ __global__ __launch_bounds__(kBlock) void fwd_attention_kernel(
     const T *__restrict__ value, const T *__restrict__ dist, const int64_t *__restrict__ shapes, int shape_stride,
     const int64_t *__restrict__ level_start, const A *__restrict__ loc, int loc_stride,
     const A *__restrict__ attn, const T *__restrict__ score_in, T *__restrict__ out, T *__restrict__ score_out,
-    A *__restrict__ weight_update, const T *__restrict__ packed, int Md, int B, int S, int M, int C, int D, int L,
+    A *__restrict__ weight_update, const T *__restrict__ packed_arg, int Md, int B, int S, int M, int C, int D, int L,
     int Q, int P, int iters, int q_blocks) {
   // packed: the head-shared distribution as dfa3d_pack_dist lays it out (D >= 2), or nullptr
   __shared__ LevelTable tab;
   __shared__ Task<A> s_tasks[kWavesPerBlock][kWave * 4];
 
   load_level_table(tab, shapes, shape_stride, level_start, L, S, FUSED ? D : 0);
-  if (FUSED && packed != nullptr) load_cell_starts(tab, L);          // uniform
+  if (FUSED && packed_arg != nullptr) load_cell_starts(tab, L);      // uniform
+  // The packed table was sized on the host for levels that share no keys (at most 2 S + 2 L cells).  A level
+  // table whose levels overlap can ask for more: then the table is not used (nor was it written) and the taps
+  // come from dist itself.
+  const T *packed = (FUSED && packed_arg != nullptr && tab.cell[L] <= packed_cell_capacity(S, L)) ? packed_arg : nullptr;
 
   const WaveShape ws = wave_shape(L, P);
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -263,6 +267,7 @@ __global__ __launch_bounds__(256) void pack_dist_kernel(
   __shared__ LevelTable tab;
   load_level_table(tab, shapes3, 3, level_start, L, S, D);
   load_cell_starts(tab, L);
+  if (tab.cell[L] > packed_cell_capacity(S, L)) return;       // overlapping levels: more cells than the table holds; the forward then ignores it
   const size_t cells = (size_t)tab.cell[L];
   const size_t n = (size_t)B * cells * D;
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {

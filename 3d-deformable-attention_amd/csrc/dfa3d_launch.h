@@ -71,12 +71,14 @@ struct BwdArgs {
   int B, S, M, C, D, L, Q, P;
   int iters;
   int vec_hint;
-  int diag;                          // development builds (-DDFA3D_EXPERIMENT) only, otherwise 0: parts of the kernels cut out
+#ifdef DFA3D_EXPERIMENT
+  int diag;                          // development builds only: parts of the kernels cut out
+  int stage;                         // development builds only: 1 binning kernels only, 2 tile kernel only
+#endif
   int tile_hint;                     // binned path: tile edge as ty * 100 + tx (0 = automatic)
   int block_hint;                    // binned path: threads per tile workgroup (0 = 512)
   int chunk_hint;                    // binned path: points of a bin per work item (0 = 4096)
   int pass_hint;                     // binned path: points per pass, 64, 128 or 256 (0 = automatic)
-  int stage;                         // development builds only, otherwise 0: 1 binning kernels only, 2 tile kernel only
   void *event_binned;                // hipEvent_t recorded between the binning kernels and the tile kernel, or nullptr
 };
 
@@ -103,6 +105,10 @@ size_t binned_depth_score_backward_workspace_bytes(const DepthScoreBwdArgs &d, i
 hipError_t launch_depth_score_backward_binned(const DepthScoreBwdArgs &d, int dtype, void *workspace,
                                               size_t workspace_bytes, int tile_hint, int chunk_hint,
                                               void *event_binned, hipStream_t stream);
+
+#ifdef DFA3D_EXPERIMENT
+size_t tile_timer_offset();
+#endif
 
 // Camera re-batching (dfa3d_rebatch.hip); strides in elements.
 hipError_t launch_rebatch_gather(const void *src, long long cam_stride, long long batch_stride, const int *index,

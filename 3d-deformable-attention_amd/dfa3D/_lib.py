@@ -111,6 +111,27 @@ def launch_options(**fields):
             _tls.fields = saved
 
 
+def current_fields():
+    """Copy of the calling thread's launch options (what an autograd Function keeps from its forward: the backward
+    of a Function with GPU inputs runs on the autograd engine's worker thread, where the caller's ``with
+    launch_options(...)`` block is not in force)."""
+    return dict(getattr(_tls, "fields", None) or {})
+
+
+@contextlib.contextmanager
+def restored_options(fields):
+    """Puts exactly ``fields`` (a dict from ``current_fields``) in force on the calling thread for the block."""
+    saved = getattr(_tls, "fields", None)
+    _tls.fields = dict(fields)
+    try:
+        yield
+    finally:
+        if saved is None:
+            del _tls.fields
+        else:
+            _tls.fields = saved
+
+
 def options():
     """ctypes argument for the ``opts`` parameter of an entry point: NULL, or the calling thread's current options."""
     fields = getattr(_tls, "fields", None)

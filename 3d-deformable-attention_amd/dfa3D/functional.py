@@ -28,10 +28,12 @@ and their ``_fp32`` / ``_fp16`` twins.  Differences from the reference, all on p
   outputs come back in bfloat16; gradients are accumulated in float32 and, in the one-kernel backward, rounded to
   bfloat16 as the tiles are written (elsewhere: float32 buffers, cast on return).
 """
+import functools
+
 import torch
 from torch.autograd.function import Function, once_differentiable
 
-from . import _ext
+from . import _ext, _lib
 
 __all__ = [
     "MultiScaleDepthScoreSampleFunction", "WeightedMultiScaleDeformableAttnFunction",
@@ -60,6 +62,18 @@ def _packed_for_forward(value_dpt_dist, value_spatial_shapes, value_level_start_
     return _ext.pack_shared_dist(value_dpt_dist, value_spatial_shapes, value_level_start_index)
 
 
+def _with_forward_options(backward):
+    """Runs a Function's backward under the launch options that were in force when its forward ran.  PyTorch calls
+    the backward of a Function with GPU inputs from the autograd engine's per-device thread, and launch options are
+    per thread: without this a ``with dfa3D._lib.launch_options(...)`` block around forward and ``.backward()``
+    would reach the forward kernels only."""
+    @functools.wraps(backward)
+    def wrapped(ctx, *grads):
+        with _lib.restored_options(getattr(ctx, "launch_fields", {})):
+            return backward(ctx, *grads)
+    return wrapped
+
+
 def _grad_in(g, like):
     """Incoming gradient as a contiguous tensor of the dtype the forward output had."""
     g = g.contiguous()
@@ -72,6 +86,7 @@ class MultiScaleDepthScoreSampleFunction(Function):
     @staticmethod
     def forward(ctx, value, value_spatial_shapes, value_level_start_index, sampling_locations, im2col_step):
         ctx.im2col_step = im2col_step
+        ctx.launch_fields = _lib.current_fields()      # the backward runs on another thread: see _with_forward_options
         output = _ext.ms_depth_score_sample_forward(
             value, value_spatial_shapes, value_level_start_index, sampling_locations,
             im2col_step=ctx.im2col_step)
@@ -80,6 +95,7 @@ class MultiScaleDepthScoreSampleFunction(Function):
 
     @staticmethod
     @once_differentiable
+    @_with_forward_options
     def backward(ctx, grad_output):
         value, value_spatial_shapes, value_level_start_index, sampling_locations = ctx.saved_tensors
         grad_value = torch.zeros(value.shape, dtype=_aux(value), device=value.device)
@@ -97,6 +113,7 @@ class WeightedMultiScaleDeformableAttnFunction(Function):
     def forward(ctx, value, value_spatial_shapes, value_level_start_index, sampling_locations,
                 attention_weights, depth_score, im2col_step):
         ctx.im2col_step = im2col_step
+        ctx.launch_fields = _lib.current_fields()      # the backward runs on another thread: see _with_forward_options
         output = _ext.wms_deform_attn_forward(
             value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights,
             depth_score, im2col_step=ctx.im2col_step)
@@ -106,6 +123,7 @@ class WeightedMultiScaleDeformableAttnFunction(Function):
 
     @staticmethod
     @once_differentiable
+    @_with_forward_options
     def backward(ctx, grad_output):
         value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights, \
             depth_score = ctx.saved_tensors
@@ -133,6 +151,7 @@ class MultiScaleDeformableAttnFunction(Function):
     def forward(ctx, value, value_spatial_shapes, value_level_start_index, sampling_locations,
                 attention_weights, im2col_step):
         ctx.im2col_step = im2col_step
+        ctx.launch_fields = _lib.current_fields()      # the backward runs on another thread: see _with_forward_options
         output = _ext.ms_deform_attn_forward(value, value_spatial_shapes, value_level_start_index,
                                              sampling_locations, attention_weights, im2col_step=ctx.im2col_step)
         ctx.save_for_backward(value, value_spatial_shapes, value_level_start_index, sampling_locations,
@@ -141,6 +160,7 @@ class MultiScaleDeformableAttnFunction(Function):
 
     @staticmethod
     @once_differentiable
+    @_with_forward_options
     def backward(ctx, grad_output):
         value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights = \
             ctx.saved_tensors
@@ -163,6 +183,7 @@ class MultiScale3DDeformableAttnFunction(Function):
     def forward(ctx, value, value_dpt_dist, value_spatial_shapes, value_level_start_index,
                 sampling_locations, attention_weights, im2col_step):
         ctx.im2col_step = im2col_step
+        ctx.launch_fields = _lib.current_fields()      # the backward runs on another thread: see _with_forward_options
         ctx.set_materialize_grads(False)
         output, depth_score = _ext.dfa3d_fused_forward(
             value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations,
@@ -175,6 +196,7 @@ class MultiScale3DDeformableAttnFunction(Function):
 
     @staticmethod
     @once_differentiable
+    @_with_forward_options
     def backward(ctx, grad_output, grad_depth_score):
         value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations, \
             attention_weights = ctx.saved_tensors
@@ -213,6 +235,7 @@ class MultiScale3DDeformableAttnWeightUpdateFunction(Function):
     def forward(ctx, value, value_dpt_dist, value_spatial_shapes, value_level_start_index,
                 sampling_locations, attention_weights, im2col_step, packed_dist=None):
         ctx.im2col_step = im2col_step
+        ctx.launch_fields = _lib.current_fields()      # the backward runs on another thread: see _with_forward_options
         ctx.set_materialize_grads(False)
         if packed_dist is None:
             packed_dist = _packed_for_forward(value_dpt_dist, value_spatial_shapes, value_level_start_index,
@@ -227,6 +250,7 @@ class MultiScale3DDeformableAttnWeightUpdateFunction(Function):
 
     @staticmethod
     @once_differentiable
+    @_with_forward_options
     def backward(ctx, grad_output, grad_weight_update):
         value, value_dpt_dist, value_spatial_shapes, value_level_start_index, sampling_locations, \
             attention_weights = ctx.saved_tensors

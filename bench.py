@@ -4,6 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload base|small|unit|dense|base_bf16|unittest|base_coherent]
     python bench.py --micro [xcd]                yardsticks of the machine (copy, bare gathers, LDS atomics, XCD map)
     python bench.py --summarize NAME DIR [DIR..] tables from rocprofv3 output directories -> profiles/NAME.txt
+    python bench.py --phase-costs [--workload W] what the parts of the backward's tile kernel cost (development build of
+                                                 the library: `python 3d-deformable-attention_amd/build.py --experiment`)
 
 A step is one forward + backward of the one-stage autograd Function
 (MultiScale3DDeformableAttnFunction.apply -> torch.autograd.grad) over one batch of synthetic
@@ -61,6 +63,9 @@ def parse():
                     help="launch option for every library call (%s)" % ", ".join(OPTION_NAMES))
     ap.add_argument("--micro", nargs="?", const="all", choices=("all", "xcd"),
                     help="run the yardstick kernels instead of the operator (xcd: only the workgroup -> XCD map)")
+    ap.add_argument("--phase-costs", action="store_true",
+                    help="time the tile kernel of the backward with parts of it cut out, and its per-phase clocks "
+                         "(needs libdfa3d_hip_experiment.so; prints a text table)")
     ap.add_argument("--summarize", nargs="+", metavar=("NAME", "DIR"),
                     help="write profiles/NAME.txt (and profiles/hbm_traffic.json) from rocprofv3 output directories")
     ap.add_argument("--summarize-command", action="append", default=[],
@@ -100,7 +105,7 @@ def recorded_traffic(workload):
 # measure library (yardstick kernels)
 # ------------------------------------------------------------------------------------------------
 def measure_lib():
-    path = os.path.join(PKG, "dfa3D", "libdfa3d_measure.so")
+    path = os.path.join(ROOT, "libdfa3d_measure.so")
     if not os.path.exists(path):
         raise ImportError(f"{path} is missing: build it with `python 3d-deformable-attention_amd/build.py`")
     h = ctypes.CDLL(path)
@@ -467,6 +472,109 @@ def cpu_baseline(w, budget_s):
                       f"OpenMP over units (forward) and over the {sample.B} batch elements (backward)"}
 
 
+# What the development build can cut out of the backward's kernels (dfa3d_experiment_set("diag", bits)), and the
+# phases thread 0 of every tile workgroup clocks (-DDFA3D_TILE_TIMING).
+PHASE_CUTS = ((0, "nothing (the kernel as shipped, with the phase clocks compiled in)"),
+              (16, "the task loop of the rows phase (dot products and weighted sums)"),
+              (512, "phase C (per-point gradients, grad_dist taps)"),
+              (2, "the grad_dist taps of phase C"),
+              (4, "the flush's device writes"),
+              (1, "the LDS tile updates of the rows phase"),
+              (256, "the grad_out row loads"),
+              (32, "the depth taps of phase A"),
+              (8, "the value row loads"),
+              (1024, "tickets (every grad_dist tap an LDS float atomic)"))
+PHASE_CLOCKS = ("item fetch", "barrier after phases A and C", "rank + staging", "scan + placement", "rows",
+                "phases A and C", "flush", "tail", "-", "-")
+
+
+def phase_costs(a):
+    """Text table: tile kernel duration with each part cut out (the difference to the first row is what that part
+    costs where it stands), and the share of thread 0's clock each phase takes."""
+    import torch
+    from dfa3D import _lib
+    _lib.LIB_PATH = os.path.join(ROOT, "libdfa3d_hip_experiment.so")
+    if not os.path.exists(_lib.LIB_PATH):
+        print("bench.py: build the development library first: python 3d-deformable-attention_amd/build.py --experiment",
+              file=sys.stderr)
+        sys.exit(3)
+    from dfa3D.workloads import WORKLOADS, make_inputs
+    L_ = _lib.lib()
+    L_.dfa3d_experiment_set.argtypes = [ctypes.c_char_p, ctypes.c_int]
+    L_.dfa3d_experiment_timer_offset.restype = ctypes.c_size_t
+    bf16 = a.workload.endswith("_bf16")
+    w = WORKLOADS["base_peaky" if a.workload == "base_bf16" else a.workload]
+    dev = torch.device("cuda:0")
+    inp = make_inputs(w, device=dev)
+    value, dist, go = inp["value"], inp["value_dpt_dist"], inp["grad_output"]
+    if bf16:
+        value, dist, go = value.bfloat16(), dist.bfloat16(), go.bfloat16()
+    shapes, lsi, loc, attn = inp["spatial_shapes"], inp["level_start_index"], inp["sampling_locations"], inp["attention_weights"]
+    B, S, M, C = value.shape
+    D = dist.shape[3]
+    _, Q, _, L, P, _ = loc.shape
+    code = _lib.dtype_code(value)
+    gv = torch.zeros(value.shape, dtype=torch.float32, device=dev)
+    gd = torch.zeros(dist.shape, dtype=torch.float32, device=dev)
+    gl, ga = torch.empty_like(loc), torch.empty_like(attn)
+    fields = {("pass_" if k == "pass" else k): int(v) for k, v in (t.split("=") for t in a.option)}
+    mid = torch.cuda.Event(enable_timing=True)
+    mid.record()
+    torch.cuda.synchronize()
+    opts = ctypes.pointer(_lib.LaunchOptions(event_binned=mid.cuda_event, **fields))
+    nbytes = L_.dfa3d_fused_backward_workspace_bytes(B, S, M, C, D, L, Q, P, M, code, opts)
+    assert nbytes > 0, "the binned backward does not take this workload"
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+
+    def call():
+        _lib.check(L_.dfa3d_fused_backward(
+            _lib.ptr(value), _lib.ptr(dist), _lib.ptr(shapes), _lib.ptr(lsi), _lib.ptr(loc), _lib.ptr(attn), _lib.ptr(go),
+            None, None, _lib.ptr(gv), _lib.ptr(gd), _lib.ptr(gl), _lib.ptr(ga), _lib.ptr(ws), nbytes, B, S, M, C, D, L, Q,
+            P, M, code, opts, _lib.stream_of(value)), "dfa3d_fused_backward")
+
+    def timed(reps):
+        bins, tiles = [], []
+        for i in range(reps + 3):
+            gv.zero_()
+            gd.zero_()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            call()
+            e1.record()
+            e1.synchronize()
+            if i >= 3:
+                bins.append(e0.elapsed_time(mid))
+                tiles.append(mid.elapsed_time(e1))
+        bins.sort()
+        tiles.sort()
+        return bins[len(bins) // 2], tiles[len(tiles) // 2]
+
+    print(f"# python bench.py --phase-costs --workload {a.workload}" + "".join(f" --option {t}" for t in a.option))
+    print(f"# development build (-DDFA3D_EXPERIMENT -DDFA3D_TILE_TIMING) of the kernel sources with digest {sources_digest()[:16]}")
+    print(f"# {torch.cuda.get_device_name(0)}; {w.points} points; medians of {a.kernel_reps} launches; a cut changes results, "
+          "its row says what the kernel takes WITHOUT that part")
+    print(f"{'cut out':72s} {'binning ms':>10s} {'tile ms':>9s} {'saves ms':>9s}")
+    base_tile = None
+    for bits, label in PHASE_CUTS:
+        L_.dfa3d_experiment_set(b"diag", bits)
+        b_ms, t_ms = timed(a.kernel_reps)
+        base_tile = t_ms if base_tile is None else base_tile
+        print(f"{label:72s} {b_ms:10.4f} {t_ms:9.4f} {base_tile - t_ms:9.4f}", flush=True)
+    L_.dfa3d_experiment_set(b"diag", 0)
+    gv.zero_()
+    gd.zero_()
+    ws.zero_()
+    call()
+    torch.cuda.synchronize()
+    off = L_.dfa3d_experiment_timer_offset()
+    ticks = ws[off:off + 80].view(torch.int64).cpu().tolist()
+    total = sum(ticks) or 1
+    print("\nshare of thread 0's clock per phase, summed over the workgroups of one launch")
+    for name, t in zip(PHASE_CLOCKS, ticks):
+        if t:
+            print(f"{name:32s} {100.0 * t / total:5.1f} %")
+
+
 def main():
     a = parse()
     if a.summarize:
@@ -486,6 +594,9 @@ def main():
         sys.exit(3)
     if a.micro:
         micro(a.micro)
+        return
+    if a.phase_costs:
+        phase_costs(a)
         return
     L_ = _lib.lib()
     user_options = {}

@@ -215,3 +215,45 @@ def test_workload_byte_model_matches_published_table():
     assert round(WORKLOADS["dense"].forward_bytes() / 1e6, 1) == 3158.8
     assert round(WORKLOADS["dense"].backward_bytes() / 1e6, 1) == 5088.8
     assert WORKLOADS["unit"].points == 12800
+
+
+def test_launch_options_follow_a_function_into_its_backward():
+    """Launch options are per thread, and PyTorch runs the backward of a Function from another thread than the one
+    that called forward (the autograd engine's device thread for GPU tensors; here: a thread of the test's own).
+    Every Function records the options its forward ran under and puts them in force again around its backward."""
+    import threading
+    import torch
+    from dfa3D import _lib, functional
+    from torch.autograd.function import Function, once_differentiable
+
+    seen = {}
+
+    class Probe(Function):
+        @staticmethod
+        def forward(ctx, x):
+            ctx.launch_fields = _lib.current_fields()
+            return x * 2
+
+        @staticmethod
+        @once_differentiable
+        @functional._with_forward_options
+        def backward(ctx, g):
+            seen["fields"] = _lib.current_fields()
+            seen["options"] = _lib.options()
+            return g * 2
+
+    x = torch.ones(3, requires_grad=True)
+    with _lib.launch_options(tile=404, **{"pass": 128}):
+        y = Probe.apply(x).sum()
+    assert _lib.options() is None                                  # the block is over on this thread
+    t = threading.Thread(target=y.backward)
+    t.start()
+    t.join()
+    assert seen["fields"] == {"tile": 404, "pass_": 128}
+    assert seen["options"] is not None and seen["options"].contents.tile == 404 and seen["options"].contents.pass_ == 128
+    assert _lib.options() is None
+    # every Function of the package is wired that way
+    for name in functional.__all__:
+        cls = getattr(functional, name)
+        base = cls.__mro__[1] if name.endswith(("_fp16", "_fp32")) else cls
+        assert hasattr(base.backward.__wrapped__, "__wrapped__"), name     # once_differentiable(_with_forward_options(backward))

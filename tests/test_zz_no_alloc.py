@@ -1,5 +1,6 @@
 """dfa3d_fused_backward_static (the backward on the library's own static scratch buffer, for callers that cannot
-allocate device memory) against dfa3d_fused_backward with a caller-provided workspace, through the C ABI."""
+allocate device memory) against dfa3d_fused_backward with a caller-provided workspace and against the CPU checker,
+through the C ABI."""
 import ctypes
 
 import pytest
@@ -37,7 +38,7 @@ def _backward(entry, ops, workspace):
     return gv, gd, gl, ga
 
 
-def test_static_scratch_backward_matches_workspace_backward():
+def test_static_scratch_backward_matches_workspace_backward(oracle):
     from dfa3D import _lib
     from dfa3D.workloads import WORKLOADS, scaled
     assert torch.cuda.is_available(), "needs the MI355X"
@@ -57,10 +58,15 @@ def test_static_scratch_backward_matches_workspace_backward():
         print("static scratch case", w.name, "needs", need, flush=True)
         want = _backward("dfa3d_fused_backward", ops, torch.empty(need, dtype=torch.uint8, device=dev))
         got = _backward("dfa3d_fused_backward_static", ops, None)
-        for name, g, x in zip(("grad_value", "grad_dist", "grad_loc", "grad_attn"), got, want):
+        cpu = [t.cpu() for t in ops]
+        _, score = oracle.dfa3d_forward(*cpu[:6])
+        checker = oracle.dfa3d_backward(*cpu[:6], score, cpu[6])
+        for name, g, x, c in zip(("grad_value", "grad_dist", "grad_loc", "grad_attn"), got, want, checker):
             assert torch.isfinite(g).all(), name
             # same kernels on the same bins: only the order of the atomic adds on tile rims differs
             torch.testing.assert_close(g, x, rtol=1e-4, atol=1e-4, msg=lambda m, n=name: f"{n}: {m}")
+            # and the float32 backward gate against the CPU checker
+            torch.testing.assert_close(g.cpu(), c, rtol=1e-4, atol=1e-4, msg=lambda m, n=name: f"{n} vs checker: {m}")
 
 
 def test_static_scratch_backward_rejects_what_does_not_fit():
