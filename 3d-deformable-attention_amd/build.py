@@ -23,9 +23,10 @@ ROOT = os.path.dirname(HERE)
 MEASURE_LIB = os.path.join(ROOT, "libdfa3d_measure.so")
 EXPERIMENT_LIB = os.path.join(ROOT, "libdfa3d_hip_experiment.so")
 EXPERIMENT_FLAGS = ["-DDFA3D_EXPERIMENT", "-DDFA3D_TILE_TIMING"]
-SOURCES = ["dfa3d_forward.hip", "dfa3d_backward.hip", "dfa3d_backward_binned.hip", "dfa3d_rebatch.hip",
+SOURCES = ["dfa3d_forward.hip", "dfa3d_backward.hip", "dfa3d_backward_binned.hip", "dfa3d_backward_cells.hip",
+           "dfa3d_rebatch.hip",
            "dfa3d_api.hip"]
-HEADERS = ["dfa3d_device.h", "dfa3d_launch.h", os.path.join("..", "..", "include", "dfa3d.h")]
+HEADERS = ["dfa3d_device.h", "dfa3d_launch.h", "dfa3d_binned.h", os.path.join("..", "..", "include", "dfa3d.h")]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",
     # keep the compiler from forming packed fp32 instructions

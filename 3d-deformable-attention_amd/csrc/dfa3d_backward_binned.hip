@@ -26,60 +26,18 @@
 //   tile_depth_backward_kernel  stage 1 alone on the same bins
 //   fill_zero / head_sum        a distribution shared by the heads: grad_dist per head, then summed
 //
-// A point belongs to the tile that holds its clamped base pixel (clamp(h0,0,H-1), clamp(w0,0,W-1)).
+// A point belongs to the tile that holds its base pixel (h0, w0) = floor of its pixel coordinates, -1 <= h0 < H,
+// -1 <= w0 < W; the tiles are laid over that range, so the first tile of a level starts at pixel -1.
 // Semantics are those of bwd_attention_kernel (see dfa3d_backward.hip for the formulas and the
 // reference lines they restate).
 #include <map>
 #include <mutex>
 #include <utility>
 
-#include "dfa3d_device.h"
-#include "dfa3d_launch.h"
+#include "dfa3d_binned.h"
 
 namespace dfa3d {
 
-constexpr int kClasses = 8;         // work queues: one per XCD (workgroup id % 8 with round-robin placement)
-constexpr int kQueueStride = 16;    // ints between queue counters: one 64-byte line each
-constexpr int kQueueInts = kClasses * kQueueStride + 32;   // + room for the optional phase timers
-constexpr int kBinQueries = 32;     // bin_points_kernel: queries of one (batch, head) per block step (16, 64, 128 time worse)
-constexpr int kHistCap = 8192;      // bins of one (batch, head) that fit the LDS histogram
-
-struct BinPlan {
-  int H[DFA3D_MAX_LEVELS], W[DFA3D_MAX_LEVELS], Dd[DFA3D_MAX_LEVELS], start[DFA3D_MAX_LEVELS];
-  int tiles_x[DFA3D_MAX_LEVELS], level_base[DFA3D_MAX_LEVELS];
-  int bins_per_bm;     // tiles over all levels of one (batch, head)
-  int total_bins;      // slots * bins_per_bm
-  int bins_per_class;  // total_bins / kClasses
-  int class_start[kClasses + 1];   // first work item of each head class (written by the scan)
-  int ty, tx;          // tile edge in pixels
-  int chunk;           // points of a bin handled by one work item
-  int total_chunks;    // work items (written by the scan)
-};
-
-// Bins are numbered slot * bins_per_bm + tile, where the slot of (batch b, head m) puts the heads with the
-// same m % 8 next to each other: class c = m % 8 owns the slots [c, c + 1) * head_groups(M) * B.  The
-// binning blocks and the tile workgroups of class c run on XCD c, so everything written and read for one
-// head (records, gradients per point, tiles) goes through one L2.
-__host__ __device__ inline int head_groups(int M) { return (M + kClasses - 1) / kClasses; }
-__host__ __device__ inline int slot_count(int B, int M) { return kClasses * head_groups(M) * B; }
-__device__ __forceinline__ int slot_of(int b, int m, int B, int M) {
-  return ((m % kClasses) * head_groups(M) + m / kClasses) * B + b;
-}
-__device__ __forceinline__ void slot_decode(int slot, int B, int M, int &b, int &m) {
-  b = slot % B;
-  const int hm = slot / B, G = head_groups(M);
-  m = (hm % G) * kClasses + hm / G;
-}
-
-struct BinWorkspace {      // device pointers into the caller's workspace
-  BinPlan *plan;
-  int *queues;             // kClasses counters, kQueueStride ints apart
-  int *counts;             // points per bin
-  int *cursor;             // begin of each bin's segment after the scan, end after the fill
-  int4 *items;             // work items: (bin, begin of its points, number of points, work items of the bin)
-  uint32_t *entries;       // point indices grouped by bin
-  float4 *recs;            // (x, y, z, attention weight) of the same points, same order
-};
 
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void plan_and_clear_kernel(
@@ -99,7 +57,9 @@ __global__ __launch_bounds__(256) void plan_and_clear_kernel(
              (D <= 0 || Dd <= D);
       }
       p.H[l] = ok ? (int)H : 0; p.W[l] = ok ? (int)W : 0; p.Dd[l] = ok ? (int)Dd : 0; p.start[l] = ok ? (int)st : 0;
-      const int nx = ok ? ((int)W + tx - 1) / tx : 0, ny = ok ? ((int)H + ty - 1) / ty : 0;
+      // tiles are laid over the base pixels of the points, which run from -1 (a location within half a pixel of
+      // the map's upper / left edge) to H - 1 / W - 1: the first tile starts at pixel -1
+      const int nx = ok ? ((int)W + tx) / tx : 0, ny = ok ? ((int)H + ty) / ty : 0;
       p.tiles_x[l] = nx;
       p.level_base[l] = base;
       base += nx * ny;
@@ -122,22 +82,10 @@ __global__ __launch_bounds__(256) void plan_and_clear_kernel(
   if (blockIdx.x == 0 && threadIdx.x < kQueueInts) ws.queues[threadIdx.x] = 0;    // the counters and their padding
 }
 
-// bin (within one (batch, head)) of a point that the operator does not skip
+// bin (within one (batch, head)) of a point that the operator does not skip: the tile that holds its base pixel
+// (h0, w0), -1 <= h0 < H, -1 <= w0 < W; tile (i, j) covers base pixels [i ty - 1, (i + 1) ty - 1) x [j tx - 1, ...)
 __device__ __forceinline__ int bin_of(const BinPlan &p, int l, const Point2D<float> &g) {
-  const int cy = min(max(g.h0, 0), p.H[l] - 1), cx = min(max(g.w0, 0), p.W[l] - 1);
-  return p.level_base[l] + (cy / p.ty) * p.tiles_x[l] + cx / p.tx;
-}
-
-// Inclusive prefix sum over the 64 lanes with DPP moves: shifts by 1, 2, 4, 8 inside rows of 16 lanes, then
-// lane 15 of a row to the next row, then lane 31 to the upper half.
-__device__ __forceinline__ int wave_inclusive_scan(int x) {
-  x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, false);   // row_shr:1
-  x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, false);   // row_shr:2
-  x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, false);   // row_shr:4
-  x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, false);   // row_shr:8
-  x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false);   // row_bcast:15 into rows 1 and 3
-  x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);   // row_bcast:31 into rows 2 and 3
-  return x;
+  return p.level_base[l] + ((g.h0 + 1) / p.ty) * p.tiles_x[l] + (g.w0 + 1) / p.tx;
 }
 
 // The fill comes in two forms.  bin_fill_sorted_kernel (few enough bins and points per unit): a block sorts its
@@ -449,8 +397,8 @@ __device__ __forceinline__ void clear_unstored(const BinWorkspace &ws, const Cle
         const int local = s - p.start[l];
         if (p.H[l] > 0 && local >= 0 && local < p.H[l] * p.W[l]) {
           const int y = local / p.W[l], x = local - y * p.W[l];
-          if (y % TY != 0 && x % TX != 0) {
-            const int bin = slot_of(b, m, B, M) * nb + p.level_base[l] + (y / TY) * p.tiles_x[l] + x / TX;
+          if ((y + 1) % TY != 0 && (x + 1) % TX != 0) {       // the first tile starts at pixel -1
+            const int bin = slot_of(b, m, B, M) * nb + p.level_base[l] + ((y + 1) / TY) * p.tiles_x[l] + (x + 1) / TX;
             const int c = ws.counts[bin];
             clear_mine = !(c > 0 && c <= ch);                 // exactly one work item: it stores this row
           }
@@ -539,18 +487,6 @@ __global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws, ClearAr
 // rims of neighbouring bins).
 // ---------------------------------------------------------------------------------------
 
-// Optional phase timing of the tile kernel (development builds only, -DDFA3D_TILE_TIMING): thread 0
-// of every workgroup accumulates shader-clock ticks per phase and adds them to 64-bit counters that
-// live in the padding behind the queue counter.
-#ifdef DFA3D_TILE_TIMING
-#define TT_DECL unsigned long long tt_acc[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long tt_last = clock64();
-#define TT_MARK(i) do { if (threadIdx.x == 0) { const unsigned long long tt_now = clock64(); tt_acc[i] += tt_now - tt_last; tt_last = tt_now; } } while (0)
-#define TT_FLUSH() do { if (threadIdx.x == 0) { unsigned long long *tt_g = reinterpret_cast<unsigned long long *>(ws.queues + kClasses * kQueueStride); for (int i = 0; i < 10; ++i) atomicAdd(tt_g + i, tt_acc[i]); } } while (0)
-#else
-#define TT_DECL
-#define TT_MARK(i) do { } while (0)
-#define TT_FLUSH() do { } while (0)
-#endif
 
 struct TileLds {      // offsets (in 4-byte words) into the dynamic LDS block
   int gv, gd, gstage, tasks, dots, cnt, offs, goff, total;
@@ -570,103 +506,9 @@ __host__ __device__ inline TileLds tile_lds_layout(int ty, int tx, int C, int D,
   return o;
 }
 
-// Thread 0 of a tile workgroup: next work item, from the queue of the workgroup's own class first and
-// from the other classes once that is empty; -1 when every queue is drained.
-__device__ __forceinline__ int pop_item(const BinWorkspace &ws, const BinPlan &p, int home, int &classes_done) {
-  while (classes_done < kClasses) {
-    const int c = (home + classes_done) % kClasses;
-    const int lo = p.class_start[c], hi = p.class_start[c + 1];
-    if (lo < hi) {
-      // from the end: the bins of the coarsest level, which hold the most points, come last in a (batch, head)
-      // and should not be what the kernel's last workgroups are left with
-      const int w = hi - 1 - atomicAdd(&ws.queues[c * kQueueStride], 1);
-      if (w >= lo) return w;
-    }
-    ++classes_done;
-  }
-  return -1;
-}
-
-// Thread 0's pipeline of work items: the item taken now was popped two items ago and its record requested
-// one item ago, so neither the queue atomic nor the record's load is waited for.
-struct ItemFetch {
-  int classes_done, w_next;
-  int4 rec;
-  __device__ __forceinline__ int4 load(const BinWorkspace &ws, int w) const {
-    return w >= 0 ? ws.items[w] : make_int4(-1, 0, 0, 0);
-  }
-  __device__ __forceinline__ void start(const BinWorkspace &ws, const BinPlan &p, int home) {
-    classes_done = 0;
-    const int w = pop_item(ws, p, home, classes_done);
-    rec = load(ws, w);
-    w_next = w >= 0 ? pop_item(ws, p, home, classes_done) : -1;
-  }
-  __device__ __forceinline__ void advance(const BinWorkspace &ws, const BinPlan &p, int home, int4 *out) {
-    *out = rec;
-    rec = load(ws, w_next);
-    w_next = w_next >= 0 ? pop_item(ws, p, home, classes_done) : -1;
-  }
-};
 
 struct RowTask { float w; uint32_t who; };   // who = point slot * 4 + corner: the index of the task's dot
 
-__device__ __forceinline__ float dpp_xadd(float x, int pick) {
-  const int xi = __float_as_int(x);
-  int r;
-  switch (pick) {
-    case 0: r = __builtin_amdgcn_mov_dpp(xi, 0xB1, 0xF, 0xF, true); break;    // quad_perm [1,0,3,2]
-    case 1: r = __builtin_amdgcn_mov_dpp(xi, 0x4E, 0xF, 0xF, true); break;    // quad_perm [2,3,0,1]
-    case 2: r = __builtin_amdgcn_mov_dpp(xi, 0x141, 0xF, 0xF, true); break;   // row_half_mirror
-    default: r = __builtin_amdgcn_mov_dpp(xi, 0x140, 0xF, 0xF, true); break;  // row_mirror
-  }
-  return x + __int_as_float(r);
-}
-template <int LPR> __device__ __forceinline__ float row_sum_f(float x) {
-  if (LPR >= 2) x = dpp_xadd(x, 0);
-  if (LPR >= 4) x = dpp_xadd(x, 1);
-  if (LPR >= 8) x = dpp_xadd(x, 2);
-  if (LPR >= 16) x = dpp_xadd(x, 3);
-  if (LPR >= 32) x += __shfl_xor(x, 16, kWave);
-  if (LPR >= 64) x += __shfl_xor(x, 32, kWave);
-  return x;
-}
-
-// VEC consecutive floats of an LDS row, moved with one instruction (the address is VEC-float
-// aligned: rows start on 16-byte boundaries and a lane's first channel is a multiple of VEC)
-template <int VEC> struct LdsVec;
-template <> struct LdsVec<1> {
-  static __device__ __forceinline__ void ld(const float *p, float (&v)[1]) { v[0] = p[0]; }
-  static __device__ __forceinline__ void st(float *p, const float (&v)[1]) { p[0] = v[0]; }
-};
-template <> struct LdsVec<2> {
-  static __device__ __forceinline__ void ld(const float *p, float (&v)[2]) {
-    const float2 t = *reinterpret_cast<const float2 *>(p);
-    v[0] = t.x; v[1] = t.y;
-  }
-  static __device__ __forceinline__ void st(float *p, const float (&v)[2]) {
-    *reinterpret_cast<float2 *>(p) = make_float2(v[0], v[1]);
-  }
-};
-template <> struct LdsVec<4> {
-  static __device__ __forceinline__ void ld(const float *p, float (&v)[4]) {
-    const float4 t = *reinterpret_cast<const float4 *>(p);
-    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-  }
-  static __device__ __forceinline__ void st(float *p, const float (&v)[4]) {
-    *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
-  }
-};
-template <> struct LdsVec<8> {
-  static __device__ __forceinline__ void ld(const float *p, float (&v)[8]) {
-    const float4 t0 = reinterpret_cast<const float4 *>(p)[0], t1 = reinterpret_cast<const float4 *>(p)[1];
-    v[0] = t0.x; v[1] = t0.y; v[2] = t0.z; v[3] = t0.w; v[4] = t1.x; v[5] = t1.y; v[6] = t1.z; v[7] = t1.w;
-  }
-  static __device__ __forceinline__ void st(float *p, const float (&v)[8]) {
-    reinterpret_cast<float4 *>(p)[0] = make_float4(v[0], v[1], v[2], v[3]);
-    reinterpret_cast<float4 *>(p)[1] = make_float4(v[4], v[5], v[6], v[7]);
-  }
-};
-template <int VEC> __device__ __forceinline__ void lds_ld(const float *p, float (&v)[VEC]) { LdsVec<VEC>::ld(p, v); }
 
 // FUSED: both stages (depth scores recomputed from dist, grad_dist and the z gradient produced).
 // !FUSED: stage 2 alone: scores read from score_in, their gradient written to grad_score_out, no
@@ -726,7 +568,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
     while (l + 1 < L && local >= p.level_base[l + 1]) ++l;
     const int tile = local - p.level_base[l];
     const int H = p.H[l], W = p.W[l], Dd = p.Dd[l], start = p.start[l];
-    const int y0 = (tile / p.tiles_x[l]) * TY, x0 = (tile % p.tiles_x[l]) * TX;
+    const int y0 = (tile / p.tiles_x[l]) * TY - 1, x0 = (tile % p.tiles_x[l]) * TX - 1;      // pixel of the tile's row 0
 
     const rsrc_t value_r = make_rsrc(value + (size_t)b * S * M * C, (size_t)S * M * C * sizeof(T));
     const int md = Md == 1 ? 0 : m;
@@ -981,7 +823,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         {
           const int r = group;
           const int y = y0 + r / TW, x = x0 + r % TW;
-          const bool ld_ok = r < R && offs[min(r, R - 1) + 1] > offs[min(r, R - 1)] && y < H && x < W && !DFA3D_DIAG(diag, 8);
+          const bool ld_ok = r < R && offs[min(r, R - 1) + 1] > offs[min(r, R - 1)] && in_map(y, x, H, W) && !DFA3D_DIAG(diag, 8);
           RowVec<T, float, VEC>::ld(value_r, (ld_ok ? (uint32_t)(((start + y * W + x) * M + m) * C * (int)sizeof(T)) : kNoRow) + chan_off, v_next);
         }
         for (int r0 = 0; r0 < R; r0 += kGroups) {        // uniform over the workgroup
@@ -993,14 +835,14 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
 #pragma unroll
           for (int off = LPR; off < kWave; off <<= 1) n_max = max(n_max, __shfl_xor(n_max, off, kWave));
           const int y = y0 + r / TW, x = x0 + r % TW;
-          const bool pix_ok = row_ok && n_r > 0 && y < H && x < W;
+          const bool pix_ok = row_ok && n_r > 0 && in_map(y, x, H, W);
           float v[VEC], acc[VEC];
 #pragma unroll
           for (int i = 0; i < VEC; ++i) { v[i] = v_next[i]; acc[i] = 0; }
           {                                              // value row of this group's next round
             const int rn = r + kGroups;
             const int yn = y0 + rn / TW, xn = x0 + rn % TW;
-            const bool ld_ok = rn < R && offs[min(rn, R - 1) + 1] > offs[min(rn, R - 1)] && yn < H && xn < W && !DFA3D_DIAG(diag, 8);
+            const bool ld_ok = rn < R && offs[min(rn, R - 1) + 1] > offs[min(rn, R - 1)] && in_map(yn, xn, H, W) && !DFA3D_DIAG(diag, 8);
             RowVec<T, float, VEC>::ld(value_r, (ld_ok ? (uint32_t)(((start + yn * W + xn) * M + m) * C * (int)sizeof(T)) : kNoRow) + chan_off, v_next);
           }
           if (DFA3D_DIAG(diag, 16)) n_max = 0;                      // cost of the task loop
@@ -1103,7 +945,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         if (nz) *reinterpret_cast<float4 *>(gv + r * C + c) = make_float4(0, 0, 0, 0);
         const int ry = r / TW, rx = r - ry * TW;
         const int y = y0 + ry, x = x0 + rx;
-        if (y < H && x < W && !DFA3D_DIAG(diag, 4)) {
+        if (in_map(y, x, H, W) && !DFA3D_DIAG(diag, 4)) {
           const uint32_t e = (uint32_t)(((start + y * W + x) * M + m) * C + c);
           const bool store = sole && ry >= 1 && ry < TY && rx >= 1 && rx < TX;
           if (store || nz) put4(gvalue_b, gvalue_r, gv16, e, val, store, true);
@@ -1116,7 +958,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         if (nz) *reinterpret_cast<float4 *>(gd + r * D + d) = make_float4(0, 0, 0, 0);
         const int ry = r / TW, rx = r - ry * TW;
         const int y = y0 + ry, x = x0 + rx;
-        if (y < H && x < W && !DFA3D_DIAG(diag, 4)) {
+        if (in_map(y, x, H, W) && !DFA3D_DIAG(diag, 4)) {
           const uint32_t e = (uint32_t)(((start + y * W + x) * Mg + mg) * D + d);
           const bool store = sole_d && ry >= 1 && ry < TY && rx >= 1 && rx < TX;
           if (store || nz) put4(gdist_b, gdist_r, gd16, e, val, store, false);
@@ -1131,7 +973,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           const int r = i / C, c = i - r * C;
           const int ry = r / TW, rx = r % TW;
           const int y = y0 + ry, x = x0 + rx;
-          if (y < H && x < W && !DFA3D_DIAG(diag, 4))
+          if (in_map(y, x, H, W) && !DFA3D_DIAG(diag, 4))
             scatter_add(gvalue_r, gvalue_f, (uint32_t)((((start + y * W + x) * M + m) * C + c) * 4), val);
         }
       }
@@ -1142,7 +984,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           const int r = i / D, d = i - r * D;
           const int ry = r / TW, rx = r % TW;
           const int y = y0 + ry, x = x0 + rx;
-          if (y < H && x < W && !DFA3D_DIAG(diag, 4))
+          if (in_map(y, x, H, W) && !DFA3D_DIAG(diag, 4))
             scatter_add(gdist_r, gdist_f, (uint32_t)((((start + y * W + x) * Mg + mg) * D + d) * 4), val);
         }
       }
@@ -1191,7 +1033,7 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
     while (l + 1 < L && local >= p.level_base[l + 1]) ++l;
     const int tile = local - p.level_base[l];
     const int H = p.H[l], W = p.W[l], Dd = p.Dd[l], start = p.start[l];
-    const int y0 = (tile / p.tiles_x[l]) * TY, x0 = (tile % p.tiles_x[l]) * TX;
+    const int y0 = (tile / p.tiles_x[l]) * TY - 1, x0 = (tile % p.tiles_x[l]) * TX - 1;      // pixel of the tile's row 0
     const rsrc_t dist_r = make_rsrc(dist + (size_t)b * S * M * D, (size_t)S * M * D * sizeof(T));
 
     // n_thr points per round (fewer than 2^16 tickets per address and round)
@@ -1260,7 +1102,7 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
         gd[i] = 0;
         const int r = i / D, d = i - r * D;
         const int y = y0 + r / TW, x = x0 + r % TW;
-        if (y < H && x < W) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * M + m) * D + d) * 4), val);
+        if (in_map(y, x, H, W)) scatter_add(gdist_r, gdist_b, (uint32_t)((((start + y * W + x) * M + m) * D + d) * 4), val);
       }
     }
   }
@@ -1270,7 +1112,8 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
 // host side
 // ---------------------------------------------------------------------------------------
 static int max_bins_per_bm(int S, int L, int ty, int tx) {
-  // tiles of a level <= (H/ty + 1) (W/tx + 1) <= HW/(ty tx) + H/ty + W/tx + 1 and H + W <= HW + 1
+  // tiles of a level = ((H + ty) / ty) ((W + tx) / tx) <= (H/ty + 1) (W/tx + 1) <= HW/(ty tx) + H/ty + W/tx + 1
+  // and H + W <= HW + 1
   const int e = ty < tx ? ty : tx;
   const long long v = (long long)S / (ty * tx) + ((long long)S + L) / e + 2LL * L + 1;
   return (int)v;
@@ -1365,7 +1208,7 @@ size_t tile_timer_offset() {
 #endif
 
 // Launch shape of the tile kernels: tile edge, threads per workgroup, points per pass.
-struct TileConfig { int ty, tx, block, pp; size_t lds; };
+struct TileConfig { int ty, tx, block, pp; size_t lds; bool cells; };      // cells: the cell-owned kernel takes the launch
 
 // kind 0: both stages, 1: stage 2 alone (no depth tile), 2: stage 1 alone (depth tile only)
 static size_t tile_lds_bytes(int kind, int ty, int tx, int C, int D, int pp) {
@@ -1383,8 +1226,26 @@ static size_t tile_lds_bytes(int kind, int ty, int tx, int C, int D, int pp) {
 //   * tiles above 8x16 pixels lose (the rows phase needs several rounds); passes of 64 points lose to 128 and 256;
 //   * an 8x8 tile at pp 128 beats a 4x8 tile at pp 256 (128 bins: 0.68 against 0.74 ms for 2.56 M points) unless
 //     most tiles take several passes (`dense`: the dense BEV workload, 41 points per pixel, 7.0 against 8.9 ms).
-static TileConfig pick_tile_config(int kind, int C, int D, int tile_hint, int block_hint, int pass_hint, bool dense) {
+static TileConfig pick_tile_config(int kind, int C, int D, int tile_hint, int block_hint, int pass_hint, bool dense,
+                                   bool cells_wanted) {
   TileConfig c;
+  c.cells = false;
+  if (cells_wanted && kind != 2 && (block_hint == 0 || block_hint == 512) && (pass_hint == 0 || pass_hint == 256)) {
+    // The cell-owned kernel (rows of 32 channels): the largest tile of at most 64 pixels whose depth tile leaves
+    // room for two workgroups per CU, else for one.
+    static const int order[][2] = {{8, 8}, {6, 8}, {4, 8}, {4, 4}, {2, 4}, {2, 2}, {1, 1}};
+    const int hy = tile_hint / 100, hx = tile_hint % 100;
+    for (size_t budget : {(size_t)79 * 1024, (size_t)150 * 1024}) {
+      for (auto &t : order) {
+        const int ty = tile_hint > 0 ? hy : t[0], tx = tile_hint > 0 ? hx : t[1];
+        const int Dk = kind == 1 ? 0 : D;
+        if (cell_kernel_applies(C, Dk, ty, tx, kind == 0) && cell_kernel_lds_bytes(ty, tx, Dk) <= budget) {
+          c.cells = true; c.block = 512; c.pp = 256; c.ty = ty; c.tx = tx; c.lds = cell_kernel_lds_bytes(ty, tx, Dk);
+          return c;
+        }
+      }
+    }
+  }
   c.block = kind == 2 ? 256 : (block_hint == 256 ? 256 : 512);
   const int pp_max = kind == 2 ? c.block : c.block / 2;      // the fused tile kernel wants two halves of pp threads
   auto clamp_pp = [&](int pp) { return pp > pp_max ? pp_max : pp; };
@@ -1423,7 +1284,8 @@ static TileConfig pick_tile_config(int kind, int C, int D, int tile_hint, int bl
 static int bwd_kind(const BwdArgs &a) { return a.dist != nullptr ? 0 : 1; }
 static TileConfig tile_config_of(const BwdArgs &a, int kind) {
   const double per_pixel = (double)a.Q * a.L * a.P / (a.S > 0 ? a.S : 1);      // sampling points per pixel of a (batch, head)
-  return pick_tile_config(kind, a.C, a.D, a.tile_hint, a.block_hint, a.pass_hint, per_pixel >= 16.0);
+  // a caller that names the channels per lane asks for the row-owned kernel, whose tiling that is
+  return pick_tile_config(kind, a.C, a.D, a.tile_hint, a.block_hint, a.pass_hint, per_pixel >= 16.0, a.vec_hint == 0);
 }
 
 static size_t workspace_bytes_for(const BwdArgs &a, int kind, int dtype) {
@@ -1470,9 +1332,8 @@ static int tile_grid(size_t lds, int block) {
   return cus * wg_per_cu;
 }
 
-template <typename K> static hipError_t allow_lds(K kern, size_t lds) {
+static hipError_t allow_lds(const void *fn, size_t lds) {
   if (lds <= 64 * 1024) return hipSuccess;
-  const void *fn = reinterpret_cast<const void *>(kern);
   const std::pair<const void *, int> key(fn, current_device());
   std::lock_guard<std::mutex> lock(g_launch_mutex);
   auto it = g_lds_allowed.find(key);
@@ -1480,6 +1341,9 @@ template <typename K> static hipError_t allow_lds(K kern, size_t lds) {
   const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e == hipSuccess) g_lds_allowed[key] = lds;
   return e;
+}
+template <typename K> static hipError_t allow_lds(K kern, size_t lds) {
+  return allow_lds(reinterpret_cast<const void *>(kern), lds);
 }
 
 template <typename T, int VEC, int LPR>
@@ -1508,9 +1372,16 @@ static hipError_t launch_tile_cfg(const BwdArgs &a, const BinWorkspace &ws, cons
   return hipGetLastError();
 }
 
+static hipError_t allow_lds(const void *fn, size_t lds);
+
 template <typename T>
 static hipError_t launch_tile_typed(const BwdArgs &a, const BinWorkspace &ws, const TileConfig &c, float *gd_heads,
                                     hipStream_t stream) {
+  if (c.cells) {
+    const int dtype = sizeof(T) == 4 ? DFA3D_F32 : DFA3D_BF16;
+    if (hipError_t e = allow_lds(cell_kernel_symbol(dtype, a.dist != nullptr), c.lds)) return e;
+    return launch_cell_kernel(a, dtype, ws, c.lds, tile_grid(c.lds, c.block), gd_heads, stream);
+  }
   // Eight channels per lane when the tile has more rows than four-channel row groups (a 9x9 tile against 64
   // groups of 8 lanes): 128 groups of 4 lanes then cover it in one round with fewer instructions per corner
   // task.  Smaller tiles would leave most of those groups idle.

@@ -475,17 +475,25 @@ def cpu_baseline(w, budget_s):
 # What the development build can cut out of the backward's kernels (dfa3d_experiment_set("diag", bits)), and the
 # phases thread 0 of every tile workgroup clocks (-DDFA3D_TILE_TIMING).
 PHASE_CUTS = ((0, "nothing (the kernel as shipped, with the phase clocks compiled in)"),
-              (16, "the task loop of the rows phase (dot products and weighted sums)"),
-              (512, "phase C (per-point gradients, grad_dist taps)"),
-              (2, "the grad_dist taps of phase C"),
+              (16, "the walk of the cells' lists / the task loop of the rows phase (dot products, weighted sums)"),
+              (512, "the per-point gradients and grad_dist taps (phase C / finish)"),
+              (2, "the grad_dist taps alone"),
               (4, "the flush's device writes"),
-              (1, "the LDS tile updates of the rows phase"),
+              (1, "the LDS tile updates of the rows phase (row-owned kernel only)"),
               (256, "the grad_out row loads"),
-              (32, "the depth taps of phase A"),
+              (32, "the depth taps of phase A / prepare"),
               (8, "the value row loads"),
               (1024, "tickets (every grad_dist tap an LDS float atomic)"))
-PHASE_CLOCKS = ("item fetch", "barrier after phases A and C", "rank + staging", "scan + placement", "rows",
-                "phases A and C", "flush", "tail", "-", "-")
+# row-owned kernel (tile_backward_kernel): thread 0's clock, ten slots
+PHASE_CLOCKS_ROWS = ("item fetch", "barrier after phases A and C", "rank + staging", "scan + placement", "rows",
+                     "phases A and C", "flush", "tail", "-", "-")
+# cell-owned kernel (cell_backward_kernel): thread 0 (a walker) fills slots 0-7, thread 256 (a pointer) slots 8-15
+PHASE_CLOCKS_CELLS = ("walker: item fetch", "walker: walk (phase X)", "walker: wait at the barrier after X",
+                      "walker: stage grad_out rows / hand over accumulators (phase Y)", "walker: wait at the barrier after Y",
+                      "-", "-", "walker: flush",
+                      "pointer: item fetch", "pointer: late grad_dist taps (phase X)", "pointer: prepare (phase X)",
+                      "pointer: wait at the barrier after X", "pointer: place (phase Y)", "pointer: finish (phase Y)",
+                      "pointer: wait at the barrier after Y", "pointer: flush")
 
 
 def phase_costs(a):
@@ -567,12 +575,16 @@ def phase_costs(a):
     call()
     torch.cuda.synchronize()
     off = L_.dfa3d_experiment_timer_offset()
-    ticks = ws[off:off + 80].view(torch.int64).cpu().tolist()
-    total = sum(ticks) or 1
-    print("\nshare of thread 0's clock per phase, summed over the workgroups of one launch")
-    for name, t in zip(PHASE_CLOCKS, ticks):
-        if t:
-            print(f"{name:32s} {100.0 * t / total:5.1f} %")
+    ticks = ws[off:off + 128].view(torch.int64).cpu().tolist()
+    cells = any(ticks[10:])                      # only the cell-owned kernel clocks more than ten slots
+    names = PHASE_CLOCKS_CELLS if cells else PHASE_CLOCKS_ROWS
+    print("\nshare of a thread's clock per phase, summed over the workgroups of one launch"
+          + (" (walkers: wavefronts 0-3, pointers: wavefronts 4-7; each role's shares add up to 100 %)" if cells else ""))
+    for lo, hi in ((0, 8), (8, 16)) if cells else ((0, 10),):
+        total = sum(ticks[lo:hi]) or 1
+        for name, t in zip(names[lo:hi], ticks[lo:hi]):
+            if t:
+                print(f"{name:72s} {100.0 * t / total:5.1f} %")
 
 
 def main():
