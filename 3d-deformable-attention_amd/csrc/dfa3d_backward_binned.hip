@@ -88,6 +88,22 @@ __device__ __forceinline__ int bin_of(const BinPlan &p, int l, const Point2D<flo
   return p.level_base[l] + ((g.h0 + 1) / p.ty) * p.tiles_x[l] + (g.w0 + 1) / p.tx;
 }
 
+// The bins of the work items decoded (batch, head, level, pixel of the tile's row 0), so that the tile workgroups
+// need no divisions to find their tile: block `block` of `n_blocks` of a fill launch takes its share of the items.
+__device__ __forceinline__ void decode_items(const BinWorkspace &ws, int B, int M, int L, int block, int n_blocks) {
+  const BinPlan &p = *ws.plan;
+  const int n = p.total_chunks;
+  for (int w = block * (int)blockDim.x + (int)threadIdx.x; w < n; w += n_blocks * (int)blockDim.x) {
+    const int bin = ws.items[w].x;
+    const int bm = bin / p.bins_per_bm, local = bin - bm * p.bins_per_bm;
+    int b, m, l = 0;
+    slot_decode(bm, B, M, b, m);
+    while (l + 1 < L && local >= p.level_base[l + 1]) ++l;
+    const int tile = local - p.level_base[l];
+    ws.geom[w] = make_int4(b | (m << 16), l, (tile / p.tiles_x[l]) * p.ty - 1, (tile % p.tiles_x[l]) * p.tx - 1);
+  }
+}
+
 // The fill comes in two forms.  bin_fill_sorted_kernel (few enough bins and points per unit): a block sorts its
 // kStage points by bin in LDS and writes each bin's run of records to consecutive addresses, so a wavefront's
 // store touches a handful of lines instead of 64.  bin_points_kernel<1>: every point's record goes straight to
@@ -110,6 +126,7 @@ __global__ __launch_bounds__(256) void bin_points_kernel(
   if (nb == 0) return;
   if (sorted_fill_applies(nb, L * P)) return;                   // bin_count_kernel / bin_fill_sorted_kernel do it
   const bool use_lds = nb <= hist_cap;
+  if (MODE == 1) decode_items(ws, B, M, L, blockIdx.x, gridDim.x);
   // The launch is a few thousand workgroups that walk the n_blocks blocks of work (so that it costs next to nothing
   // when the kernel steps aside).  head = block % M: with the round-robin placement of workgroups on the 8 XCDs
   // and a grid that is a multiple of 8, the records of one (batch, head) are written through one XCD's L2.
@@ -257,6 +274,7 @@ __global__ __launch_bounds__(kFillThreads) void bin_fill_sorted_kernel(
   const int nb = p.bins_per_bm;
   const int LP = L * P;
   if (nb == 0 || !sorted_fill_applies(nb, LP)) return;
+  decode_items(ws, B, M, L, blockIdx.x, gridDim.x);
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int m = blockIdx.x % M, rest = blockIdx.x / M;          // head = block % M, as in bin_points_kernel
   const int qb = rest % q_blocks, b = rest / q_blocks;
@@ -1178,7 +1196,7 @@ __global__ __launch_bounds__(256) void head_sum_kernel(const float *__restrict__
     }
   }
 }
-struct BinLayout { size_t plan, queues, counts, cursor, items, entries, recs, gd_heads, total; };
+struct BinLayout { size_t plan, queues, counts, cursor, items, geom, entries, recs, gd_heads, total; };
 static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
   BinLayout o;
   const size_t nbins = (size_t)max_bins_per_bm(a.S, a.L, ty, tx) * slot_count(a.B, a.M);
@@ -1190,7 +1208,8 @@ static BinLayout bin_layout(const BwdArgs &a, int ty, int tx) {
   o.cursor = up(o.counts + nbins * sizeof(int));
   // work items: at most one partial chunk per bin plus the full chunks
   o.items = up(o.cursor + nbins * sizeof(int));
-  o.entries = up(o.items + (nbins + npts / kMinChunk + 1) * sizeof(int4));
+  o.geom = up(o.items + (nbins + npts / kMinChunk + 1) * sizeof(int4));
+  o.entries = up(o.geom + (nbins + npts / kMinChunk + 1) * sizeof(int4));
   o.recs = up(o.entries + npts * sizeof(uint32_t));
   // a distribution shared by the heads: grad_dist per head first (stores, as with a distribution per head),
   // summed over the heads afterwards; eight XCDs adding atomically into one shared tile cost twice as much
@@ -1406,6 +1425,7 @@ static BinWorkspace carve_workspace(void *workspace, const BinLayout &lay) {
   ws.counts = reinterpret_cast<int *>(base + lay.counts);
   ws.cursor = reinterpret_cast<int *>(base + lay.cursor);
   ws.items = reinterpret_cast<int4 *>(base + lay.items);
+  ws.geom = reinterpret_cast<int4 *>(base + lay.geom);
   ws.entries = reinterpret_cast<uint32_t *>(base + lay.entries);
   ws.recs = reinterpret_cast<float4 *>(base + lay.recs);
   return ws;

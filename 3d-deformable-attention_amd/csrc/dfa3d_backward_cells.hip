@@ -33,7 +33,10 @@ constexpr int kCellBlock = 512;       // threads: wavefronts 0-3 walk, 4-7 own t
 constexpr int kCellPass = 256;        // points per pass: one per pointer thread
 constexpr int kCellC = 32;            // channels: 4 lanes of 8
 constexpr int kCellMax = 64;          // cells per tile: 4 walker wavefronts of 16 groups
-constexpr int kGPitch = kCellC;       // words between staged grad_out rows
+#ifndef DFA3D_CELL_GPITCH
+#define DFA3D_CELL_GPITCH 32
+#endif
+constexpr int kGPitch = DFA3D_CELL_GPITCH;       // words between staged grad_out rows
 // the row of zeros behind the staged rows must also lie behind the accumulators that take their place when an item ends
 static_assert(kCellMax * 4 * kCellC <= kCellPass * kGPitch, "accumulators would overwrite the row of zeros");
 
@@ -76,16 +79,58 @@ struct PointState {
   uint32_t gp;                // index of the point
   float a, sc[4], hl[4];      // attention weight; corner scores; upper minus lower depth tap per corner
   float lh, lw, ld;           // fractional parts along h, w, depth
-  int d0;                     // lower depth bin
-  uint32_t tr01, tr23;        // tile rows of the corners, 16 bits each, 0xFFFF = none
-  unsigned bits;              // bit k: corner k inside the map; 4: depth inside; 5, 6: lower, upper tap exists; 7: live
+  unsigned bits;              // bit k: corner k inside the map; 4: depth inside; 5, 6: lower, upper tap exists; 7: live;
+                              // 8-13: the point's cell; 16-31: lower depth bin + 1
 };
 // the taps of a finished point that found their address taken: added atomically one phase later
 struct LateTaps {
-  float v[8];                 // value of tap j (corner j / 2, lower / upper bin)
-  int at[4];                  // tile address of each corner's lower tap, -1 = none
-  unsigned late;              // bit j: tap j is still to be added
+  float gs[4], hd, ld;        // gradient at each corner's score; weights of the lower and the upper bin
+  unsigned pack;              // bit j: tap j (corner j / 2, lower / upper bin) is still to be added; 8-13: cell; 16-31: lower bin + 1
 };
+// Queue state of the thread that fetches the work items: the item taken now was popped two items ago and its two
+// records asked for one item ago, so neither the queue atomic nor the loads are waited for.
+struct CellFetch {
+  int classes_done, w_next;
+  int4 rec, geo;
+  __device__ __forceinline__ void load(const BinWorkspace &ws, int w) {
+    rec = w >= 0 ? ws.items[w] : make_int4(-1, 0, 0, 0);
+    geo = w >= 0 ? ws.geom[w] : make_int4(0, 0, 0, 0);
+  }
+  __device__ __forceinline__ void start(const BinWorkspace &ws, const BinPlan &p, int home) {
+    classes_done = 0;
+    const int w = pop_item(ws, p, home, classes_done);
+    load(ws, w);
+    w_next = w >= 0 ? pop_item(ws, p, home, classes_done) : -1;
+  }
+  __device__ __forceinline__ void advance(const BinWorkspace &ws, const BinPlan &p, int home, int4 *r, int4 *g) {
+    *r = rec; *g = geo;
+    load(ws, w_next);
+    w_next = w_next >= 0 ? pop_item(ws, p, home, classes_done) : -1;
+  }
+};
+// a work item, decoded
+struct ItemGeom { int bin, seg, n_item, chunks, b, m, H, W, Dd, start, y0, x0; };
+// an item record read from LDS is the same in every lane: keep it in scalar registers
+__device__ __forceinline__ ItemGeom uniform(const ItemGeom &g) {
+  ItemGeom u;
+  u.bin = __builtin_amdgcn_readfirstlane(g.bin); u.seg = __builtin_amdgcn_readfirstlane(g.seg);
+  u.n_item = __builtin_amdgcn_readfirstlane(g.n_item); u.chunks = __builtin_amdgcn_readfirstlane(g.chunks);
+  u.b = __builtin_amdgcn_readfirstlane(g.b); u.m = __builtin_amdgcn_readfirstlane(g.m);
+  u.H = __builtin_amdgcn_readfirstlane(g.H); u.W = __builtin_amdgcn_readfirstlane(g.W);
+  u.Dd = __builtin_amdgcn_readfirstlane(g.Dd); u.start = __builtin_amdgcn_readfirstlane(g.start);
+  u.y0 = __builtin_amdgcn_readfirstlane(g.y0); u.x0 = __builtin_amdgcn_readfirstlane(g.x0);
+  return u;
+}
+
+// Four partial sums per lane (one per corner) over the four lanes of a group: lane c gets the whole sum of corner c.
+// Two exchange steps in which every lane passes on the two (then one) partial sums its partner collects.
+__device__ __forceinline__ float quad_corner_sum(float d0, float d1, float d2, float d3, bool odd, bool upper) {
+  const float keep_a = odd ? d1 : d0, send_a = odd ? d0 : d1, keep_b = odd ? d3 : d2, send_b = odd ? d2 : d3;
+  const float a = keep_a + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(send_a), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+  const float b = keep_b + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(send_b), 0xB1, 0xF, 0xF, true));
+  const float keep = upper ? b : a, send = upper ? a : b;
+  return keep + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(send), 0x4E, 0xF, 0xF, true));               // quad_perm [2,3,0,1]
+}
 
 // FUSED: both stages (depth scores recomputed from dist, grad_dist and the z gradient produced).
 // !FUSED: stage 2 alone: scores read from score_in, their gradient written to grad_score_out, no depth tile
@@ -101,7 +146,9 @@ __global__ __launch_bounds__(kCellBlock, 4) void cell_backward_kernel(
   // Md: heads stored in dist (M, or 1 = shared by all heads); Mg: heads of the grad_dist buffer written here
   constexpr int C = kCellC, PP = kCellPass, VEC = 8, LPR = 4;
   extern __shared__ __align__(16) float smem[];
-  __shared__ int4 s_item;
+  __shared__ int s_lv[4][DFA3D_MAX_LEVELS];              // the plan's level tables: H, W, Dd, first key
+  __shared__ CellFetch s_fetch;                           // the fetching thread's queue state, between its turns
+  __shared__ ItemGeom s_geom[3];                         // the item before, this one and the next, decoded by the thread that fetches them
 
   const BinPlan &p = *ws.plan;
   const int nb = p.bins_per_bm;
@@ -124,106 +171,221 @@ __global__ __launch_bounds__(kCellBlock, 4) void cell_backward_kernel(
   const int cell = wave * (kWave / LPR) + lane / LPR;      // walkers: the cell of this lane group
   const int LP = L * P;
   const int n_bit_words = (R * D + 31) / 32;
+  const bool gv16 = (grad16 & 1) != 0, gd16 = (grad16 & 2) != 0;          // uniform
 
   for (int i = tid; i < lay.gstage; i += kCellBlock) smem[i] = 0;                   // depth tile and bitmap
-  for (int i = tid; i < C; i += kCellBlock) gstage[PP * kGPitch + i] = 0;           // the row idle lanes read
   for (int i = tid; i < 2 * kCellMax; i += kCellBlock) cnt[i] = 0;
+  if (tid < DFA3D_MAX_LEVELS) {      // decoding an item then costs no dependent loads from device memory
+    s_lv[0][tid] = p.H[tid]; s_lv[1][tid] = p.W[tid]; s_lv[2][tid] = p.Dd[tid]; s_lv[3][tid] = p.start[tid];
+  }
+  __syncthreads();
   CT_DECL
 
-  ItemFetch fetch;
-  if (tid == 0) fetch.start(ws, p, blockIdx.x % kClasses);
-  for (;;) {
-    // ---- next work item: (bin, chunk of its points), in bin order
-    __syncthreads();
-    if (tid == 0) fetch.advance(ws, p, blockIdx.x % kClasses, &s_item);
-    __syncthreads();
-    const int4 item = s_item;
-    const int bin = item.x, seg = item.y, n_item = item.z, chunks_here = item.w;
-    if (bin < 0) break;                                   // queues drained: every wave leaves
-    CT_MARK(0);
-    const int bm = bin / nb, local = bin - bm * nb;
-    int b, m;
-    slot_decode(bm, B, M, b, m);
-    int l = 0;
-    while (l + 1 < L && local >= p.level_base[l + 1]) ++l;
-    const int tile = local - p.level_base[l];
-    const int H = p.H[l], W = p.W[l], Dd = p.Dd[l], start = p.start[l];
-    const int y0 = (tile / p.tiles_x[l]) * TY - 1, x0 = (tile % p.tiles_x[l]) * TX - 1;      // pixel of the tile's row 0
-    const int n_pass = (n_item + PP - 1) / PP;
-
-    if (walker) {
-      // =========================== walkers ===========================
-      const rsrc_t value_r = make_rsrc(value + (size_t)b * S * M * C, (size_t)S * M * C * sizeof(T));
-      const rsrc_t go_r = make_rsrc(grad_out + (size_t)b * Q * M * C, (size_t)Q * M * C * sizeof(T));
-      const uint32_t chan_off = (uint32_t)(cl * VEC * sizeof(T));
-      // the four value rows of this group's cell (zero outside the map, or when the cell is not part of the tile)
-      float v[4][VEC], acc[4][VEC];
-      {
-        const int cy = cell / TX, cx = cell - cy * TX;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const int y = y0 + cy + (k >= 2 ? 1 : 0), x = x0 + cx + ((k == 1 || k == 2) ? 1 : 0);
-          const bool ok = cell < n_cells && in_map(y, x, H, W) && !DFA3D_DIAG(diag, 8);
-          RowVec<T, float, VEC>::ld(value_r, (ok ? (uint32_t)(((start + y * W + x) * M + m) * C * (int)sizeof(T)) : kNoRow) + chan_off, v[k]);
-#pragma unroll
-          for (int i = 0; i < VEC; ++i) acc[k][i] = 0;
-        }
+  // four consecutive elements at element index `e` of a batch slice of a gradient: stored, or added atomically
+  auto put4 = [&](char *base, rsrc_t r, bool is16, uint32_t e, const float4 &val, bool store, bool every) {
+    if (!is16) {
+      float *fb = reinterpret_cast<float *>(base);
+      if (store) {
+        *reinterpret_cast<float4 *>(fb + e) = val;                              // zeros too: full lines
+      } else {
+        if (every || val.x != 0) scatter_add(r, fb, e * 4, val.x);
+        if (every || val.y != 0) scatter_add(r, fb, e * 4 + 4, val.y);
+        if (every || val.z != 0) scatter_add(r, fb, e * 4 + 8, val.z);
+        if (every || val.w != 0) scatter_add(r, fb, e * 4 + 12, val.w);
       }
-      for (int turn = 0; turn <= n_pass + 1; ++turn) {      // uniform over the workgroup
-        // ---------------- phase X: walk the lists of pass turn - 1 ----------------
-        for (int i = tid; i < n_bit_words; i += 4 * kWave) bitmap[i] = 0;          // last used in phase Y before
-        if (turn >= 1) {
-          int *c_old = cnt + ((turn - 1) & 1) * kCellMax;                          // the sort of pass turn - 1 is over
-          if (tid < kCellMax) c_old[tid] = 0;
-        }
-        if (turn >= 1 && turn <= n_pass && !DFA3D_DIAG(diag, 16)) {
-          const int beg = cell < n_cells ? offs[cell] : 0, end = cell < n_cells ? offs[cell + 1] : 0;
-          constexpr int UT = 2;
-          const float *g_lane = gstage + cl * VEC;
-          for (int t = beg; t < end; t += UT) {
-            int sl[UT];
-            float4 w4[UT];
-            float gg[UT][VEC];
+    } else {
+      char *dst = base + (size_t)e * 2;
+      if (store) {
+        *reinterpret_cast<uint2 *>(dst) = make_uint2(pack_bf16x2(val.x, val.y), pack_bf16x2(val.z, val.w));
+      } else {
+        if (val.x != 0 || val.y != 0) atomic_add_bf16x2(dst, val.x, val.y);
+        if (val.z != 0 || val.w != 0) atomic_add_bf16x2(dst + 4, val.z, val.w);
+      }
+    }
+  };
+
+  // The depth tile of the item in slot `which` goes out and is left zeroed: threads first, first + step, ... of the
+  // float4 groups (both roles share the work in the one phase in which nobody adds to the tile).
+  auto flush_gd = [&](int which, int first, int step) {
+const ItemGeom q = uniform(s_geom[which]);
+    const int mg = Mg == 1 ? 0 : q.m;
+    char *gdist_b = static_cast<char *>(grad_dist) + (size_t)q.b * S * Mg * D * (gd16 ? 2 : 4);
+    const rsrc_t gdist_r = make_rsrc(gdist_b, (size_t)S * Mg * D * sizeof(float));
+    const bool sole_d = q.chunks == 1 && Mg == M;       // a gradient shared by the heads collects from all of them
+    const int d4n = D >> 2;
+    for (int i0 = first; i0 < R * d4n; i0 += step) {
+      int i = i0;
+      asm volatile("" : "+v"(i));                 // not to be worked out ahead of the loop and kept in registers
+      const int r = i / d4n, d = (i - r * d4n) << 2;
+      float4 val = *reinterpret_cast<float4 *>(gd + r * D + d);
+      const bool nz = val.x != 0 || val.y != 0 || val.z != 0 || val.w != 0;
+      if (nz) *reinterpret_cast<float4 *>(gd + r * D + d) = make_float4(0, 0, 0, 0);
+      const int ry = r / TW, rx = r - ry * TW;
+      const int y = q.y0 + ry, x = q.x0 + rx;
+      if (in_map(y, x, q.H, q.W) && !DFA3D_DIAG(diag, 4)) {
+        const uint32_t e = (uint32_t)(((q.start + y * q.W + x) * Mg + mg) * D + d);
+        const bool store = sole_d && ry >= 1 && ry < TY && rx >= 1 && rx < TX;
+        if (store || nz) put4(gdist_b, gdist_r, gd16, e, val, store, false);
+      }
+    }
+  };
+  // Work items follow one another without a pause.  An item of n passes takes n + 1 turns of two phases (X, Y: one
+  // barrier after each); what is left of it when its last turn ends is dealt with beside the first turns of the item
+  // after it: its accumulators (handed over in LDS in its last phase Y) go out in phase X of turn 0, the late taps of
+  // its last pass come in that same phase, and its depth tile goes out in phase X of turn 1, before the new item's
+  // first finish touches the tile.  When the queues are drained one more item of zero passes does the same for the
+  // last real one.
+  //   X(t)  walkers: t = 0: value rows of the item, accumulators of the item before; else walk pass t - 1
+  //         pointers: late taps of the pass finished last; prepare pass t; t = 1: depth tile of the item before
+  //   Y(t)  walkers: stage pass t, or (t = n) hand over the accumulators
+  //         pointers: place pass t; finish pass t - 1; ask for the records of the next pass
+  // The two roles run the same sequence of items, turns and barriers, each in a loop of its own: what a role keeps in
+  // registers from turn to turn then never competes with the other role's registers.
+  if (walker) {
+    // =========================== walkers ===========================
+    float v[4][VEC], acc[4][VEC];
 #pragma unroll
-            for (int j = 0; j < UT; ++j) {
-              const bool on = t + j < end;
-              const int idx = min(t + j, PP - 1);
-              const int s = s_slot[idx];
-              const float4 w = s_w[idx];
-              sl[j] = on ? s : PP;                              // an idle step reads the row of zeros, weight zero
-              w4[j] = on ? w : make_float4(0, 0, 0, 0);
+    for (int k = 0; k < 4; ++k) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) { v[k][i] = 0; acc[k][i] = 0; }
+    }
+    const uint32_t chan_off = (uint32_t)(cl * VEC * sizeof(T));
+    auto decode = [&](const int4 &item, const int4 &geo) {
+      ItemGeom g;
+      g.bin = item.x; g.seg = item.y; g.n_item = item.z; g.chunks = item.w;
+      g.b = geo.x & 0xFFFF; g.m = geo.x >> 16;
+      const int l = geo.y;
+      g.H = s_lv[0][l]; g.W = s_lv[1][l]; g.Dd = s_lv[2][l]; g.start = s_lv[3][l];
+      g.y0 = geo.z; g.x0 = geo.w;                            // pixel of the tile's row 0
+      return g;
+    };
+    if (tid == 0) {
+      CellFetch fetch;
+      int4 rec, geo;
+      fetch.start(ws, p, blockIdx.x % kClasses);
+      fetch.advance(ws, p, blockIdx.x % kClasses, &rec, &geo);
+      s_geom[0] = decode(rec, geo);
+      s_fetch = fetch;
+    }
+    __syncthreads();                                        // the first item's record is there
+    for (int it = 0;; ++it) {
+      const ItemGeom g = uniform(s_geom[it % 3]);
+      const bool have_prev = it > 0, done = g.bin < 0;
+      if (done && !have_prev) break;
+      const int n_pass = done ? 0 : (g.n_item + PP - 1) / PP;
+      CT_MARK(0);
+      // The record of the item after this one, first of all: here the walkers hold nothing in registers (the
+      // accumulators were handed over, the value rows are about to be replaced), and nobody reads the slot before
+      // this item's last phase Y.
+      if (tid == 0 && !done) {
+        CellFetch fetch = s_fetch;
+        int4 rec, geo;
+        fetch.advance(ws, p, blockIdx.x % kClasses, &rec, &geo);
+        s_geom[(it + 1) % 3] = decode(rec, geo);
+        s_fetch = fetch;
+      }
+      const rsrc_t value_r = make_rsrc(value + (size_t)g.b * S * M * C, (size_t)S * M * C * sizeof(T));
+      const rsrc_t go_r = make_rsrc(grad_out + (size_t)g.b * Q * M * C, (size_t)Q * M * C * sizeof(T));
+      for (int turn = 0; turn <= n_pass; ++turn) {          // uniform over the workgroup
+        // ---------------- phase X ----------------
+        for (int i = tid; i < n_bit_words; i += PP) bitmap[i] = 0;                 // last used in the phase Y before
+        if (turn >= 1 && tid < kCellMax) cnt[((turn - 1) & 1) * kCellMax + tid] = 0;   // the sort of pass turn - 1 is over
+        if (turn == 0) {
+          // the four value rows of this group's cell (zero outside the map, or when the cell is not part of the
+          // tile), asked for first: they arrive while the accumulators of the item before go out
+          {
+            const int cy = cell / TX, cx = cell - cy * TX;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const int y = g.y0 + cy + (k >= 2 ? 1 : 0), x = g.x0 + cx + ((k == 1 || k == 2) ? 1 : 0);
+              const bool ok = !done && cell < n_cells && in_map(y, x, g.H, g.W) && !DFA3D_DIAG(diag, 8);
+              RowVec<T, float, VEC>::ld(value_r, (ok ? (uint32_t)(((g.start + y * g.W + x) * M + g.m) * C * (int)sizeof(T)) : kNoRow) + chan_off, v[k]);
             }
+          }
+          if (have_prev) {
+            // Pixel (ry, rx) of the tile collects corner 0 of cell (ry, rx), corner 1 of (ry, rx - 1), corner 2 of
+            // (ry - 1, rx - 1) and corner 3 of (ry - 1, rx), four floats per lane.  Pixels 1..TY-1 x 1..TX-1 belong to
+            // no neighbour's halo; when the item held all the points of its bin nobody else adds to them, so they are
+            // stored instead of added atomically (grad_value is zero on entry, or the binning launches cleared what is
+            // added to).
+            const ItemGeom q = uniform(s_geom[(it + 2) % 3]);
+            char *gvalue_b = static_cast<char *>(grad_value) + (size_t)q.b * S * M * C * (gv16 ? 2 : 4);
+            const rsrc_t gvalue_r = make_rsrc(gvalue_b, (size_t)S * M * C * sizeof(float));
+            constexpr int c4n = C >> 2;
+            for (int i0 = tid; i0 < R * c4n; i0 += PP) {
+              int i = i0;
+              asm volatile("" : "+v"(i));             // not to be worked out ahead of the loop and kept in registers
+              const int r = i / c4n, c = (i - r * c4n) << 2;
+              const int ry = r / TW, rx = r - ry * TW;
+              float4 val = make_float4(0, 0, 0, 0);
 #pragma unroll
-            for (int j = 0; j < UT; ++j) lds_ld<VEC>(g_lane + sl[j] * kGPitch, gg[j]);
+              for (int k = 0; k < 4; ++k) {
+                const int cy = ry - (k >= 2 ? 1 : 0), cx = rx - ((k == 1 || k == 2) ? 1 : 0);
+                if (cy >= 0 && cy < TY && cx >= 0 && cx < TX) {
+                  const float4 t = *reinterpret_cast<const float4 *>(gstage + ((cy * TX + cx) * 4 + k) * C + c);
+                  val.x += t.x; val.y += t.y; val.z += t.z; val.w += t.w;
+                }
+              }
+              const bool nz = val.x != 0 || val.y != 0 || val.z != 0 || val.w != 0;
+              const int y = q.y0 + ry, x = q.x0 + rx;
+              if (in_map(y, x, q.H, q.W) && !DFA3D_DIAG(diag, 4)) {
+                const uint32_t e = (uint32_t)(((q.start + y * q.W + x) * M + q.m) * C + c);
+                const bool store = q.chunks == 1 && ry >= 1 && ry < TY && rx >= 1 && rx < TX;
+                if (store || nz) put4(gvalue_b, gvalue_r, gv16, e, val, store, true);
+              }
+            }
+          }
 #pragma unroll
-            for (int j = 0; j < UT; ++j) {
+          for (int k = 0; k < 4; ++k) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[k][i] = 0;
+          }
+        } else if (!DFA3D_DIAG(diag, 16)) {
+          // walk the lists of pass turn - 1
+          const int beg = cell < n_cells ? offs[cell] : 0, end = cell < n_cells ? offs[cell + 1] : 0;
+          if (beg < end) {                                  // lanes leave the loop as their cell's list ends
+            // One point per step; the next step's grad_out row is asked for while this step's sums are formed, so
+            // that no LDS round trip is waited for with nothing to do.
+            const float *g_lane = gstage + cl * VEC;
+            int s_cur = s_slot[beg];
+            float g_cur[VEC];
+            lds_ld<VEC>(g_lane + s_cur * kGPitch, g_cur);
+            for (int t = beg; t < end; ++t) {
+              const int s_nxt = s_slot[t + 1 < end ? t + 1 : t];
+              const float4 w_cur = s_w[t];
               float d[4];
 #pragma unroll
               for (int k = 0; k < 4; ++k) {
                 d[k] = 0;
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) d[k] += v[k][i] * gg[j][i];
+                for (int i = 0; i < VEC; ++i) d[k] += v[k][i] * g_cur[i];
               }
-#pragma unroll
-              for (int k = 0; k < 4; ++k) d[k] = row_sum_f<LPR>(d[k]);
-              const float wk[4] = {w4[j].x, w4[j].y, w4[j].z, w4[j].w};
+              float g_nxt[VEC];
+              lds_ld<VEC>(g_lane + s_nxt * kGPitch, g_nxt);
+              const float wk[4] = {w_cur.x, w_cur.y, w_cur.z, w_cur.w};
 #pragma unroll
               for (int k = 0; k < 4; ++k) {
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) acc[k][i] += wk[k] * gg[j][i];
+                for (int i = 0; i < VEC; ++i) acc[k][i] += wk[k] * g_cur[i];
               }
-              // lane c of the group reports corner c's dot; an idle step's goes to a scrap word
-              const float mine_d = cl == 0 ? d[0] : cl == 1 ? d[1] : cl == 2 ? d[2] : d[3];
-              dots[sl[j] < PP ? sl[j] * 4 + cl : PP * 4 + lane] = mine_d;
+              dots[s_cur * 4 + cl] = quad_corner_sum(d[0], d[1], d[2], d[3], (cl & 1) != 0, (cl & 2) != 0);   // lane c reports corner c
+              s_cur = s_nxt;
+#pragma unroll
+              for (int i = 0; i < VEC; ++i) g_cur[i] = g_nxt[i];
             }
           }
         }
+        if (turn == 1) {
+          // the depth tile of the item before: complete since the late taps of turn 0, not touched again before this
+          // item's first finish in phase Y of this turn
+          if (FUSED && have_prev) flush_gd((it + 2) % 3, tid, kCellBlock);
+        }
         CT_MARK(1);
-        __syncthreads();
+        lds_barrier();
         CT_MARK(2);
-        if (turn > n_pass) break;
-        // ---------------- phase Y: stage the grad_out rows of pass turn ----------------
+        // ---------------- phase Y ----------------
         if (turn < n_pass) {
+          // stage the grad_out rows of pass turn
           constexpr int RPI = kWave / LPR, kRows = PP / 4;      // rows per load instruction, rows per walker wavefront
 #pragma unroll
           for (int j = 0; j < kRows; j += RPI) {
@@ -233,6 +395,8 @@ __global__ __launch_bounds__(kCellBlock, 4) void cell_backward_kernel(
             RowVec<T, float, VEC>::ld(go_r, goff[slot] + chan_off, gg);
             LdsVec<VEC>::st(gstage + slot * kGPitch + cl * VEC, gg);
           }
+        } else if (done) {
+          if (FUSED && have_prev) flush_gd((it + 2) % 3, tid, PP);   // the last item's depth tile: nothing follows
         } else {
           // the item's last walk is over: the cells' accumulators go where the staged rows were
           if (cell < n_cells) {
@@ -241,59 +405,82 @@ __global__ __launch_bounds__(kCellBlock, 4) void cell_backward_kernel(
           }
         }
         CT_MARK(3);
-        __syncthreads();
+        lds_barrier();
         CT_MARK(4);
       }
-    } else {
-      // =========================== pointers ===========================
-      const int md = Md == 1 ? 0 : m;
-      const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)b * S * Md * D : nullptr, FUSED ? (size_t)S * Md * D * sizeof(T) : 0);
-      PointState cur, nxt;
-      LateTaps late;
-      cur.bits = 0; nxt.bits = 0; late.late = 0;
-      cur.gp = nxt.gp = 0; cur.a = nxt.a = 0; cur.lh = cur.lw = cur.ld = nxt.lh = nxt.lw = nxt.ld = 0; cur.d0 = nxt.d0 = 0;
-      cur.tr01 = cur.tr23 = nxt.tr01 = nxt.tr23 = 0xFFFFFFFFu;
+      if (done) break;
+    }
+  } else {
+    // =========================== pointers ===========================
+    PointState cur, nxt;
+    LateTaps late;
+    uint32_t pre_gp = 0;                                    // index and record of the point this thread prepares next
+    float4 pre_rec = make_float4(0, 0, 0, 0);
+    cur.bits = 0; nxt.bits = 0; late.pack = 0; late.hd = late.ld = 0;
+    cur.gp = nxt.gp = 0; cur.a = nxt.a = 0; cur.lh = cur.lw = cur.ld = nxt.lh = nxt.lw = nxt.ld = 0;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) { cur.sc[k] = cur.hl[k] = nxt.sc[k] = nxt.hl[k] = 0; late.at[k] = -1; }
+    for (int k = 0; k < 4; ++k) { cur.sc[k] = cur.hl[k] = nxt.sc[k] = nxt.hl[k] = 0; late.gs[k] = 0; }
+    __syncthreads();                                        // the first item's record is there
+    {
+      const ItemGeom g0 = uniform(s_geom[0]);
+      if (g0.bin >= 0 && pslot < g0.n_item) {
+        pre_gp = ws.entries[g0.seg + pslot];
+        pre_rec = ws.recs[g0.seg + pslot];
+      }
+    }
+    for (int it = 0;; ++it) {
+      const ItemGeom g = uniform(s_geom[it % 3]);
+      const bool have_prev = it > 0, done = g.bin < 0;
+      if (done && !have_prev) break;
+      const int n_pass = done ? 0 : (g.n_item + PP - 1) / PP;
+      CT_MARK(0);
+      const int md = Md == 1 ? 0 : g.m;
+      const rsrc_t dist_r = make_rsrc(FUSED ? dist + (size_t)g.b * S * Md * D : nullptr, FUSED ? (size_t)S * Md * D * sizeof(T) : 0);
+      const rsrc_t go_r = make_rsrc(grad_out + (size_t)g.b * Q * M * C, (size_t)Q * M * C * sizeof(T));
+      for (int turn = 0; turn <= n_pass; ++turn) {          // uniform over the workgroup
+        // ---------------- phase X: late taps of the pass finished last, then prepare pass turn ----------------
+        if (FUSED && (late.pack & 0xFFu)) {
+          const int lcell = (late.pack >> 8) & 63, lcy = lcell / TX, lcx = lcell - lcy * TX, ld0 = (int)(late.pack >> 16) - 1;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) late.v[j] = 0;
-      for (int turn = 0; turn <= n_pass + 1; ++turn) {      // uniform over the workgroup
-        // ---------------- phase X: late taps of pass turn - 2, then prepare pass turn ----------------
-        if (FUSED && late.late) {
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-            if (late.late >> j & 1) atomicAdd(gd + late.at[j >> 1] + (j & 1), late.v[j]);
-          late.late = 0;
+          for (int j = 0; j < 8; ++j) {
+            if (late.pack >> j & 1) {
+              const int k = j >> 1, row = (lcy + (k >= 2 ? 1 : 0)) * TW + lcx + ((k == 1 || k == 2) ? 1 : 0);
+              atomicAdd(gd + row * D + ld0 + (j & 1), ((j & 1) ? late.ld : late.hd) * late.gs[k]);
+            }
+          }
+          late.pack = 0;
         }
         CT_MARK(1);
-        float4 pw = make_float4(0, 0, 0, 0);               // corner weights in the order of the cell's corners
+        float4 pw = make_float4(0, 0, 0, 0);               // corner weights of this thread's point
         int my_cell = -1, my_rank = 0;
         if (turn < n_pass) {
           const int base = turn * PP;
-          const bool live = pslot < n_item - base;
-          Point2D<float> g;
+          const bool live = pslot < g.n_item - base;
+          Point2D<float> pg;
           DepthTap<float> tap;
           size_t gp = 0;
           float a = 0, wk[4] = {0, 0, 0, 0};
-          int tr[4] = {-1, -1, -1, -1};
           unsigned on_bits = 0;
 #pragma unroll
-          for (int k = 0; k < 4; ++k) { nxt.sc[k] = 0; nxt.hl[k] = 0; g.key[k] = -1; }
-          g.inside = false; g.lh = g.lw = g.hh = g.hw = 0; g.h0 = g.w0 = 0;
+          for (int k = 0; k < 4; ++k) { nxt.sc[k] = 0; nxt.hl[k] = 0; pg.key[k] = -1; }
+          pg.inside = false; pg.lh = pg.lw = pg.hh = pg.hw = 0; pg.h0 = pg.w0 = 0;
           tap.inside = tap.lo_ok = tap.hi_ok = false; tap.d0 = 0; tap.ld = tap.hd = 0;
-          uint32_t my_goff = kNoRow;
+          uint32_t my_goff = kNoRow, touch = 0;
           if (live) {
-            gp = ws.entries[seg + base + pslot];
-            const float4 rec = ws.recs[seg + base + pslot];
+            gp = pre_gp;                                     // asked for one phase ago
+            const float4 rec = pre_rec;
             const size_t unit = gp / LP;
             a = rec.w;
-            g = locate_2d<float>(rec.x, rec.y, H, W, start);
+            my_goff = (uint32_t)((unit - (size_t)g.b * Q * M) * C * sizeof(T));
+            // ask for the point's grad_out row now, so that the walkers' staging loads of the next phase find it in the L2
+            touch = __builtin_amdgcn_raw_buffer_load_b32(go_r, my_goff, 0, 0);
+            pg = locate_2d<float>(rec.x, rec.y, g.H, g.W, g.start);
             if (FUSED) {
-              tap = locate_depth<float>(rec.z, Dd);
+              tap = locate_depth<float>(rec.z, g.Dd);
               if (DFA3D_DIAG(diag, 32)) { for (int k = 0; k < 4; ++k) { nxt.sc[k] = 0.5f; nxt.hl[k] = 0.1f; } } else   // cost of the depth taps
               {
                 float lo[4], hi[4];
-                corner_scores<T, float, true>(dist_r, g.key, tap, md, Md, D, nxt.sc, lo, hi);
+                corner_scores<T, float, true>(dist_r, pg.key, tap, md, Md, D, nxt.sc, lo, hi);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) nxt.hl[k] = hi[k] - lo[k];
               }
@@ -302,37 +489,31 @@ __global__ __launch_bounds__(kCellBlock, 4) void cell_backward_kernel(
 #pragma unroll
               for (int k = 0; k < 4; ++k) nxt.sc[k] = score_in != nullptr ? Elem<T>::ld(si + k) : 1.f;
             }
-            my_goff = (uint32_t)((unit - (size_t)b * Q * M) * C * sizeof(T));
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-              if (g.key[k] >= 0) {
+              if (pg.key[k] >= 0) {
                 on_bits |= 1u << k;
-                const int ry = g.h0 + (k >= 2 ? 1 : 0) - y0, rx = g.w0 + ((k == 1 || k == 2) ? 1 : 0) - x0;
-                if (ry >= 0 && ry <= TY && rx >= 0 && rx <= TX) {
-                  tr[k] = ry * TW + rx;
-                  wk[k] = g.bil(k) * nxt.sc[k] * a;
-                }
+                wk[k] = pg.bil(k) * nxt.sc[k] * a;
               }
             }
-            if (g.inside) {
+            if (pg.inside) {
               // the cell: the base pixel within the tile (the binning put the point into this tile by it)
-              const int cy = min(max(g.h0 - y0, 0), TY - 1), cx = min(max(g.w0 - x0, 0), TX - 1);
+              const int cy = min(max(pg.h0 - g.y0, 0), TY - 1), cx = min(max(pg.w0 - g.x0, 0), TX - 1);
               my_cell = cy * TX + cx;
               my_rank = atomicAdd(cnt + (turn & 1) * kCellMax + my_cell, 1);
             }
           }
+          if (touch == 0x7FC12345u) my_goff = kNoRow;      // never (a NaN payload no gradient carries): keeps the load alive
           goff[pslot] = my_goff;
           pw = make_float4(wk[0], wk[1], wk[2], wk[3]);
-          nxt.gp = (uint32_t)gp; nxt.a = a; nxt.lh = g.lh; nxt.lw = g.lw; nxt.ld = tap.ld; nxt.d0 = tap.d0;
-          nxt.tr01 = ((uint32_t)tr[0] & 0xFFFFu) | ((uint32_t)tr[1] << 16);
-          nxt.tr23 = ((uint32_t)tr[2] & 0xFFFFu) | ((uint32_t)tr[3] << 16);
+          nxt.gp = (uint32_t)gp; nxt.a = a; nxt.lh = pg.lh; nxt.lw = pg.lw; nxt.ld = tap.ld;
           nxt.bits = on_bits | (tap.inside ? 16u : 0u) | (tap.lo_ok ? 32u : 0u) | (tap.hi_ok ? 64u : 0u) |
-                     ((live && my_cell >= 0) ? 128u : 0u);
+                     ((live && my_cell >= 0) ? 128u : 0u) | ((unsigned)max(my_cell, 0) << 8) | ((unsigned)(tap.d0 + 1) << 16);
         }
+        if (FUSED && have_prev && turn == 1) flush_gd((it + 2) % 3, tid, kCellBlock);     // the walkers take the other half
         CT_MARK(2);
-        __syncthreads();
+        lds_barrier();
         CT_MARK(3);
-        if (turn > n_pass) break;
         // ---------------- phase Y: place pass turn, finish pass turn - 1 ----------------
         if (turn < n_pass) {
           // exclusive prefix of the cell counters; every pointer wavefront computes it and writes the same numbers,
@@ -349,30 +530,28 @@ __global__ __launch_bounds__(kCellBlock, 4) void cell_backward_kernel(
         }
         CT_MARK(4);
         if (turn >= 1 && (cur.bits & 128u) && !DFA3D_DIAG(diag, 512)) {       // (development builds: cost of phase C)
-          Point2D<float> g;
+          Point2D<float> pg;
           DepthTap<float> tap;
-          g.lh = cur.lh; g.lw = cur.lw; g.hh = 1 - cur.lh; g.hw = 1 - cur.lw;
+          pg.lh = cur.lh; pg.lw = cur.lw; pg.hh = 1 - cur.lh; pg.hw = 1 - cur.lw;
           tap.inside = (cur.bits & 16u) != 0; tap.lo_ok = (cur.bits & 32u) != 0; tap.hi_ok = (cur.bits & 64u) != 0;
-          tap.d0 = cur.d0; tap.ld = cur.ld; tap.hd = tap.inside ? 1 - cur.ld : 0.f;
-          int trc[4] = {(int)(int16_t)(cur.tr01 & 0xFFFFu), (int)(int16_t)(cur.tr01 >> 16),
-                        (int)(int16_t)(cur.tr23 & 0xFFFFu), (int)(int16_t)(cur.tr23 >> 16)};
+          tap.d0 = (int)(cur.bits >> 16) - 1; tap.ld = cur.ld; tap.hd = tap.inside ? 1 - cur.ld : 0.f;
           const unsigned on_bits = cur.bits & 15u;
+          const int ccell = (cur.bits >> 8) & 63, ccy = ccell / TX, ccx = ccell - ccy * TX;
           const float a = cur.a;
           const size_t gp = cur.gp;
           const float4 d4 = *reinterpret_cast<const float4 *>(dots + pslot * 4);
           const float dc[4] = {d4.x, d4.y, d4.z, d4.w};
-          float gs[4], s[4], ga = 0;
+          float gs[4], sk[4], ga = 0;
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
-            const float dk = dc[k];
             const bool on = on_bits >> k & 1;
-            const float bk = g.bil(k);
-            gs[k] = on ? bk * a * dk : 0.f;
-            s[k] = on ? cur.sc[k] * dk : 0.f;
-            ga += bk * s[k];
+            const float bk = pg.bil(k);
+            gs[k] = on ? bk * a * dc[k] : 0.f;
+            sk[k] = on ? cur.sc[k] * dc[k] : 0.f;
+            ga += bk * sk[k];
           }
-          const float gx = (float)W * a * (g.hh * (s[1] - s[0]) + g.lh * (s[2] - s[3]));
-          const float gy = (float)H * a * (g.hw * (s[3] - s[0]) + g.lw * (s[2] - s[1]));
+          const float gx = (float)g.W * a * (pg.hh * (sk[1] - sk[0]) + pg.lh * (sk[2] - sk[3]));
+          const float gy = (float)g.H * a * (pg.hw * (sk[3] - sk[0]) + pg.lw * (sk[2] - sk[1]));
           float *gl = grad_loc + gp * gl_stride;
           if (!FUSED) { gl[0] = gx; gl[1] = gy; }
           if (FUSED) {
@@ -389,19 +568,20 @@ __global__ __launch_bounds__(kCellBlock, 4) void cell_backward_kernel(
             }
             float gz = 0;
             unsigned want = 0;                          // bit j: tap j exists
+            int at4[4];                                 // tile address of each corner's lower tap
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-              const bool corner_in = (on_bits >> k & 1) && tap.inside;
-              const bool taps = trc[k] >= 0 && tap.inside && gs[k] != 0 && !DFA3D_DIAG(diag, 2);
-              late.at[k] = taps ? trc[k] * D + tap.d0 : -1;
+              const bool corner_in = (on_bits >> k & 1) && tap.inside;     // a corner inside the map lies inside the tile
+              if (!corner_in) gs[k] = 0.f;
+              const bool taps = corner_in && gs[k] != 0 && !DFA3D_DIAG(diag, 2);
+              at4[k] = ((ccy + (k >= 2 ? 1 : 0)) * TW + ccx + ((k == 1 || k == 2) ? 1 : 0)) * D + tap.d0;
               if (taps && tap.lo_ok) want |= 1u << (2 * k);
               if (taps && tap.hi_ok) want |= 2u << (2 * k);
-              if (!corner_in) gs[k] = 0.f;
               gz += gs[k] * cur.hl[k];
-              late.v[2 * k] = tap.hd * gs[k];
-              late.v[2 * k + 1] = tap.ld * gs[k];
+              late.gs[k] = gs[k];
             }
-            gl[0] = gx; gl[1] = gy; gl[2] = gz * (float)Dd;      // one 12-byte store
+            late.hd = tap.hd; late.ld = tap.ld;
+            gl[0] = gx; gl[1] = gy; gl[2] = gz * (float)g.Dd;      // one 12-byte store
             grad_attn[gp] = ga;                       // all stores before the tile updates: they complete slowly
             // Who is first at a tile address in this pass: the bit of the address in the bitmap, set with an integer
             // atomic.  The first adds at once with a plain read-modify-write (nobody else touches the address before
@@ -410,18 +590,18 @@ __global__ __launch_bounds__(kCellBlock, 4) void cell_backward_kernel(
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
               if (want >> j & 1) {
-                const int at = late.at[j >> 1] + (j & 1);
+                const int at = at4[j >> 1] + (j & 1);
                 const uint32_t bit = 1u << (at & 31);
                 if (DFA3D_DIAG(diag, 1024) || (atomicOr(&bitmap[at >> 5], bit) & bit)) {} else first |= 1u << j;
               }
             }
             float cur8[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) cur8[j] = (first >> j & 1) ? gd[late.at[j >> 1] + (j & 1)] : 0.f;
+            for (int j = 0; j < 8; ++j) cur8[j] = (first >> j & 1) ? gd[at4[j >> 1] + (j & 1)] : 0.f;
 #pragma unroll
             for (int j = 0; j < 8; ++j)
-              if (first >> j & 1) gd[late.at[j >> 1] + (j & 1)] = cur8[j] + late.v[j];
-            late.late = want & ~first;
+              if (first >> j & 1) gd[at4[j >> 1] + (j & 1)] = cur8[j] + ((j & 1) ? tap.ld : tap.hd) * gs[j >> 1];
+            late.pack = (want & ~first) | (cur.bits & 0xFFFF3F00u);
           } else if (grad_score_out != nullptr) {
             float *go4 = grad_score_out + gp * 4;
 #pragma unroll
@@ -431,90 +611,26 @@ __global__ __launch_bounds__(kCellBlock, 4) void cell_backward_kernel(
             grad_attn[gp] = ga;
           }
         }
+        // the records of the next pass's points (of this item, or of the first pass of the item after it, whose record
+        // was written in phase X of turn 1): they arrive while the workgroup waits at the barrier
+        if (!done) {
+          const bool last = turn >= n_pass;
+          const ItemGeom ng = uniform(s_geom[(it + 1) % 3]);
+          const int next_seg = last ? ng.seg : g.seg, next_base = last ? 0 : (turn + 1) * PP;
+          const int next_n = last ? (ng.bin >= 0 ? ng.n_item : 0) : g.n_item;
+          if ((!last || turn >= 1) && pslot < next_n - next_base) {
+            pre_gp = ws.entries[next_seg + next_base + pslot];
+            pre_rec = ws.recs[next_seg + next_base + pslot];
+          }
+        }
         cur = nxt;
         nxt.bits = 0;
         CT_MARK(5);
-        __syncthreads();
+        lds_barrier();
         CT_MARK(6);
       }
+      if (done) break;
     }
-    // Both roles have passed the same barriers; the last one came after the late taps of the final pass, so the
-    // depth tile is complete, and the cells' accumulators lie in LDS.
-
-    // ---------------- flush the tile (and leave the depth tile zeroed for the next item) ----------------
-    const bool gv16 = (grad16 & 1) != 0, gd16 = (grad16 & 2) != 0;          // uniform
-    const int mg = Mg == 1 ? 0 : m;
-    char *gvalue_b = static_cast<char *>(grad_value) + (size_t)b * S * M * C * (gv16 ? 2 : 4);
-    char *gdist_b = FUSED ? static_cast<char *>(grad_dist) + (size_t)b * S * Mg * D * (gd16 ? 2 : 4) : nullptr;
-    const rsrc_t gvalue_r = make_rsrc(gvalue_b, (size_t)S * M * C * sizeof(float));
-    const rsrc_t gdist_r = make_rsrc(gdist_b, FUSED ? (size_t)S * Mg * D * sizeof(float) : 0);
-    // Pixels 1..TY-1 x 1..TX-1 of the tile belong to no neighbour's halo; when this item holds all the
-    // points of its bin nobody else adds to them, so they are stored instead of added atomically
-    // (grad_value and grad_dist are zero on entry).
-    const bool sole = chunks_here == 1;
-    const bool sole_d = sole && Mg == M;                 // a gradient shared by the heads collects from all of them
-    // four consecutive elements at element index `e` of a batch slice: stored, or added atomically
-    auto put4 = [&](char *base, rsrc_t r, bool is16, uint32_t e, const float4 &val, bool store, bool every) {
-      if (!is16) {
-        float *fb = reinterpret_cast<float *>(base);
-        if (store) {
-          *reinterpret_cast<float4 *>(fb + e) = val;                              // zeros too: full lines
-        } else {
-          if (every || val.x != 0) scatter_add(r, fb, e * 4, val.x);
-          if (every || val.y != 0) scatter_add(r, fb, e * 4 + 4, val.y);
-          if (every || val.z != 0) scatter_add(r, fb, e * 4 + 8, val.z);
-          if (every || val.w != 0) scatter_add(r, fb, e * 4 + 12, val.w);
-        }
-      } else {
-        char *dst = base + (size_t)e * 2;
-        if (store) {
-          *reinterpret_cast<uint2 *>(dst) = make_uint2(pack_bf16x2(val.x, val.y), pack_bf16x2(val.z, val.w));
-        } else {
-          if (val.x != 0 || val.y != 0) atomic_add_bf16x2(dst, val.x, val.y);
-          if (val.z != 0 || val.w != 0) atomic_add_bf16x2(dst + 4, val.z, val.w);
-        }
-      }
-    };
-    // grad_value: pixel (ry, rx) of the tile collects corner 0 of cell (ry, rx), corner 1 of (ry, rx - 1), corner 2
-    // of (ry - 1, rx - 1) and corner 3 of (ry - 1, rx), four floats per lane
-    constexpr int c4n = C >> 2;
-    const int d4n = D >> 2;
-    for (int i = tid; i < R * c4n; i += kCellBlock) {
-      const int r = i / c4n, c = (i - r * c4n) << 2;
-      const int ry = r / TW, rx = r - ry * TW;
-      float4 val = make_float4(0, 0, 0, 0);
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int cy = ry - (k >= 2 ? 1 : 0), cx = rx - ((k == 1 || k == 2) ? 1 : 0);
-        if (cy >= 0 && cy < TY && cx >= 0 && cx < TX) {
-          const float4 t = *reinterpret_cast<const float4 *>(gstage + ((cy * TX + cx) * 4 + k) * C + c);
-          val.x += t.x; val.y += t.y; val.z += t.z; val.w += t.w;
-        }
-      }
-      const bool nz = val.x != 0 || val.y != 0 || val.z != 0 || val.w != 0;
-      const int y = y0 + ry, x = x0 + rx;
-      if (in_map(y, x, H, W) && !DFA3D_DIAG(diag, 4)) {
-        const uint32_t e = (uint32_t)(((start + y * W + x) * M + m) * C + c);
-        const bool store = sole && ry >= 1 && ry < TY && rx >= 1 && rx < TX;
-        if (store || nz) put4(gvalue_b, gvalue_r, gv16, e, val, store, true);
-      }
-    }
-    if (FUSED) {
-      for (int i = tid; i < R * d4n; i += kCellBlock) {
-        const int r = i / d4n, d = (i - r * d4n) << 2;
-        float4 val = *reinterpret_cast<float4 *>(gd + r * D + d);
-        const bool nz = val.x != 0 || val.y != 0 || val.z != 0 || val.w != 0;
-        if (nz) *reinterpret_cast<float4 *>(gd + r * D + d) = make_float4(0, 0, 0, 0);
-        const int ry = r / TW, rx = r - ry * TW;
-        const int y = y0 + ry, x = x0 + rx;
-        if (in_map(y, x, H, W) && !DFA3D_DIAG(diag, 4)) {
-          const uint32_t e = (uint32_t)(((start + y * W + x) * Mg + mg) * D + d);
-          const bool store = sole_d && ry >= 1 && ry < TY && rx >= 1 && rx < TX;
-          if (store || nz) put4(gdist_b, gdist_r, gd16, e, val, store, false);
-        }
-      }
-    }
-    CT_MARK(7);
   }
   CT_FLUSH();
 }

@@ -44,12 +44,22 @@ __device__ __forceinline__ void slot_decode(int slot, int B, int M, int &b, int 
 // pixel (y, x) lies inside an H x W map (a tile's first row and column may be pixel -1)
 __device__ __forceinline__ bool in_map(int y, int x, int H, int W) { return (unsigned)y < (unsigned)H && (unsigned)x < (unsigned)W; }
 
+// Workgroup barrier that orders LDS accesses only.  __syncthreads() also waits for every global load and store the
+// wavefront has in flight (one counter covers both on this part); the tile workgroups hand work to each other
+// through LDS alone, so their loads may stay in flight across a barrier and their stores may drain behind it.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 struct BinWorkspace {      // device pointers into the caller's workspace
   BinPlan *plan;
   int *queues;             // kClasses counters, kQueueStride ints apart
   int *counts;             // points per bin
   int *cursor;             // begin of each bin's segment after the scan, end after the fill
   int4 *items;             // work items: (bin, begin of its points, number of points, work items of the bin)
+  int4 *geom;              // the items' bins decoded: (batch | head << 16, level, pixel row, pixel column of the tile's row 0)
   uint32_t *entries;       // point indices grouped by bin
   float4 *recs;            // (x, y, z, attention weight) of the same points, same order
 };
