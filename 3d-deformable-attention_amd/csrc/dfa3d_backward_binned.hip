@@ -38,6 +38,12 @@
 
 namespace dfa3d {
 
+#ifdef DFA3D_TILE_SYNCTHREADS
+#define TILE_BARRIER() __syncthreads()
+#else
+#define TILE_BARRIER() lds_barrier()
+#endif
+
 
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void plan_and_clear_kernel(
@@ -572,9 +578,9 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
   int pass_tag = 0x5EED0000;                               // changes with every pass of this workgroup
   for (;;) {
     // ---- next work item: (bin, chunk of its points), in bin order
-    __syncthreads();
+    TILE_BARRIER();
     if (tid == 0) fetch.advance(ws, p, blockIdx.x % kClasses, &s_item);
-    __syncthreads();
+    TILE_BARRIER();
     const int4 item = s_item;
     const int bin = item.x, seg = item.y, n_item = item.z, chunks_here = item.w;
     if (bin < 0) break;                                   // queues drained: every wave leaves
@@ -764,7 +770,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
         }
       }
       if (ticketed && pass_idx > 0) {
-        __syncthreads();                                 // plain updates done before the atomic ones start
+        TILE_BARRIER();                                 // plain updates done before the atomic ones start
         if (prev_mine && live) {
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
@@ -778,7 +784,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
       }
       TT_MARK(5);
       if (!has) break;
-      __syncthreads();                                   // counters cleared, goff visible
+      TILE_BARRIER();                                   // counters cleared, goff visible
       TT_MARK(1);
       int rank[4];
 #pragma unroll
@@ -800,7 +806,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           if (slot_ok && chan < C) LdsVec<VEC>::st(gstage + slot * C + chan, gg);
         }
       }
-      __syncthreads();                                   // counts complete
+      TILE_BARRIER();                                   // counts complete
       TT_MARK(2);
       // Exclusive prefix of the row counters.  Every wavefront that places tasks computes it, two rows per
       // lane and 128 rows per step, and writes the same numbers: it can go on with its own copy without
@@ -829,7 +835,7 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           dots[slot * 4 + k] = 0;                        // no row will write this dot
         }
       }
-      __syncthreads();                                   // tasks grouped by row, grad_out rows staged
+      TILE_BARRIER();                                   // tasks grouped by row, grad_out rows staged
       TT_MARK(3);
 
       // ---------------- rows: one group of LPR lanes per tile row ----------------
@@ -914,10 +920,10 @@ __global__ __launch_bounds__(512, 4) void tile_backward_kernel(
           }
         }
       }
-      __syncthreads();                                   // dots complete
+      TILE_BARRIER();                                   // dots complete
       TT_MARK(4);
     }
-    __syncthreads();                                     // the tile is complete
+    TILE_BARRIER();                                     // the tile is complete
 
     // ---------------- flush the tile (and leave it zeroed for the next item) ----------------
     const bool gv16 = (grad16 & 1) != 0, gd16 = (grad16 & 2) != 0;          // uniform
@@ -1038,9 +1044,9 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
   ItemFetch fetch;
   if (tid == 0) fetch.start(ws, p, blockIdx.x % kClasses);
   for (;;) {
-    __syncthreads();
+    TILE_BARRIER();
     if (tid == 0) fetch.advance(ws, p, blockIdx.x % kClasses, &s_item);
-    __syncthreads();
+    TILE_BARRIER();
     const int4 item = s_item;
     const int bin = item.x, seg = item.y, n_item = item.z;
     if (bin < 0) break;                                   // queues drained: every wave leaves
@@ -1093,7 +1099,7 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
         float *gl = grad_loc3 + gp * 3;
         gl[0] = 0; gl[1] = 0; gl[2] = gz * (float)Dd;
       }
-      __syncthreads();                                     // every ticket of the round taken
+      TILE_BARRIER();                                     // every ticket of the round taken
       uint16_t *ticket16 = reinterpret_cast<uint16_t *>(tickets);
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
@@ -1102,7 +1108,7 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
           if (first_mask & (2u << (2 * k))) { gd[at[k]] += tap.ld * gk[k]; ticket16[at[k]] = 0; }
         }
       }
-      __syncthreads();                                     // plain updates done before the atomic ones start
+      TILE_BARRIER();                                     // plain updates done before the atomic ones start
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         if (at[k] >= 0) {
@@ -1111,7 +1117,7 @@ __global__ __launch_bounds__(256) void tile_depth_backward_kernel(
         }
       }
     }
-    __syncthreads();
+    TILE_BARRIER();
     float *gdist_b = grad_dist + (size_t)b * S * M * D;
     const rsrc_t gdist_r = make_rsrc(gdist_b, (size_t)S * M * D * sizeof(float));
     for (int i = tid; i < R * D; i += n_thr) {

@@ -24,7 +24,7 @@ class Workload:
     P: int                      # sampling points per level
     M: int = 8                  # heads
     C: int = 32                 # channels per head
-    loc: str = "uniform"        # "uniform" in [lo, hi]^3, "normal" clipped to [lo, hi], or "coherent" (see make_inputs)
+    loc: str = "uniform"        # "uniform" in [lo, hi]^3, "normal" clipped to [lo, hi], "coherent" or "band" (see make_inputs)
     loc_lo: float = 0.0
     loc_hi: float = 1.0
     loc_mean: float = 0.5
@@ -52,18 +52,19 @@ class Workload:
             acc += h * w
         return out
 
-    def forward_bytes(self, e_v=4, e_o=4):
-        """Algorithmic bytes of one forward: every operand read once, every result written once."""
+    def forward_bytes(self, e_v=4, e_o=4, e_a=4):
+        """Algorithmic bytes of one forward: every operand read once, every result written once.  e_v, e_o, e_a:
+        bytes per element of value / dist, of output / depth_score, of locations / attention weights."""
         n = self.points
-        return (e_v * self.B * self.S * self.M * (self.C + self.D) + 16 * n + 4 * e_o * n
+        return (e_v * self.B * self.S * self.M * (self.C + self.D) + 4 * e_a * n + 4 * e_o * n
                 + e_o * self.B * self.Q * self.M * self.C)
 
-    def backward_bytes(self, e_v=4, e_o=4):
+    def backward_bytes(self, e_v=4, e_o=4, e_a=4):
         """Algorithmic bytes of one backward (saved depth_score re-read, zero fills excluded)."""
         n = self.points
-        reads = (e_v * self.B * self.S * self.M * (self.C + self.D) + 16 * n + 4 * e_o * n
+        reads = (e_v * self.B * self.S * self.M * (self.C + self.D) + 4 * e_a * n + 4 * e_o * n
                  + e_o * self.B * self.Q * self.M * self.C)
-        writes = e_v * self.B * self.S * self.M * (self.C + self.D) + 16 * n
+        writes = e_v * self.B * self.S * self.M * (self.C + self.D) + 4 * e_a * n
         return reads + writes
 
 
@@ -88,12 +89,19 @@ WORKLOADS = {
     # (spatial_cross_attention.py:505-538: reference point + offset / (W, H, D))
     "base_coherent": Workload("base_coherent", B=6, Q=10000, levels=_BASE_LEVELS, D=64, P=8, depth_sigma=2.0,
                               loc="coherent", loc_std=0.02),
+    # Two probes of the forward kernel's cache behaviour at the base shape.  base_coarse: the three coarse levels
+    # alone, whose value rows and distributions of one (batch, head) fit an XCD's L2 (2.9 MB).  base_band: all four
+    # levels, but the locations of level 0 confined to the upper third of the map, i.e. what a forward that walks
+    # level 0 band by band would find in the L2 during one band.
+    "base_coarse": Workload("base_coarse", B=6, Q=10000, levels=_BASE_LEVELS[1:], D=64, P=8, depth_sigma=2.0),
+    "base_band": Workload("base_band", B=6, Q=10000, levels=_BASE_LEVELS, D=64, P=8, depth_sigma=2.0, loc="band"),
     # dense BEV grid, clustered locations
     "dense": Workload("dense", B=6, Q=40000, levels=_BASE_LEVELS, D=128, P=8, loc="normal",
                       loc_lo=-0.1, loc_hi=1.1, depth_sigma=2.0),
 }
 
-SEEDS = {"unit": 1, "small": 2, "base": 3, "base_peaky": 4, "dense": 5, "unittest": 6, "base_coherent": 7}
+SEEDS = {"unit": 1, "small": 2, "base": 3, "base_peaky": 4, "dense": 5, "unittest": 6, "base_coherent": 7,
+         "base_coarse": 3, "base_band": 3}
 
 
 def scaled(w: Workload, B=None, Q=None, name=None) -> Workload:
@@ -132,6 +140,8 @@ def make_inputs(w: Workload, seed=None, dtype=torch.float32, device="cpu", grad_
         loc = torch.randn(B, Q, M, L, P, 3, generator=g, dtype=torch.float32) * spread + centre.view(1, Q, 1, 1, 1, 3)
     else:
         loc = torch.rand(B, Q, M, L, P, 3, generator=g, dtype=torch.float32) * (w.loc_hi - w.loc_lo) + w.loc_lo
+        if w.loc == "band":
+            loc[:, :, :, 0, :, 1] /= 3.0                     # level 0: rows of the upper third of the map only
     if w.attn == "rand":
         attn = torch.rand(B, Q, M, L, P, generator=g, dtype=torch.float32)
     else:

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the DFA3D operator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload base|small|unit|dense|base_bf16|unittest|base_coherent]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload base|small|unit|dense|base_bf16|base_f64|unittest|base_coherent]
     python bench.py --micro [xcd]                yardsticks of the machine (copy, bare gathers, LDS atomics, XCD map)
     python bench.py --summarize NAME DIR [DIR..] tables from rocprofv3 output directories -> profiles/NAME.txt
     python bench.py --phase-costs [--workload W] what the parts of the backward's tile kernel cost (development build of
@@ -218,6 +218,7 @@ def micro(sections="all"):
 # rocprofv3 summaries
 # ------------------------------------------------------------------------------------------------
 KERNEL_KEYS = (("fwd_attention_kernel", "forward"), ("tile_backward_kernel", "backward_tile"),
+               ("cell_backward_kernel", "backward_tile"),
                ("bin_fill_sorted_kernel", "bin_fill"), ("bin_count_kernel", "bin_count"),
                ("bin_scan_kernel", "bin_scan_and_clear"))
 
@@ -269,8 +270,8 @@ def summarize(name, dirs, commands):
     for path in [d for d in dirs if d.endswith(".json")]:
         lines += summarize_json(path)
     dirs = [d for d in dirs if not d.endswith(".json")]
-    cols = ("fwd_attention_kernel", "tile_backward_kernel", "bin_count_kernel", "bin_fill_sorted_kernel",
-            "stream_copy_kernel")
+    cols = ("fwd_attention_kernel", "cell_backward_kernel", "tile_backward_kernel", "bin_count_kernel",
+            "bin_fill_sorted_kernel", "stream_copy_kernel")
     for d in dirs:
         for db in sorted(glob.glob(os.path.join(d, "**", "*.db"), recursive=True)):
             c = sqlite3.connect(db)
@@ -623,19 +624,22 @@ def main():
 
 
 def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
-    bf16 = a.workload.endswith("_bf16")
-    wname = "base_peaky" if a.workload == "base_bf16" else a.workload
+    bf16, f64 = a.workload.endswith("_bf16"), a.workload.endswith("_f64")
+    wname = "base_peaky" if a.workload == "base_bf16" else a.workload[:-4] if f64 else a.workload
     w = WORKLOADS[wname]
     dev = torch.device("cuda:0")
     inp = make_inputs(w, device=dev)
+    if f64:         # the other type the reference dispatches (wms_deform_attn_cuda.cu:267): the device-atomics kernels
+        inp = {k: (v.double() if v.is_floating_point() else v) for k, v in inp.items()}
     value, dist = inp["value"], inp["value_dpt_dist"]
     go = inp["grad_output"]
     if bf16:
         value, dist, go = value.bfloat16(), dist.bfloat16(), go.bfloat16()
     shapes, lsi = inp["spatial_shapes"], inp["level_start_index"]
     loc, attn = inp["sampling_locations"], inp["attention_weights"]
-    e_v = 2 if bf16 else 4
-    fwd_bytes, bwd_bytes = w.forward_bytes(e_v, e_v), w.backward_bytes(e_v, e_v)
+    e_v = 2 if bf16 else 8 if f64 else 4
+    e_a = 8 if f64 else 4
+    fwd_bytes, bwd_bytes = w.forward_bytes(e_v, e_v, e_a), w.backward_bytes(e_v, e_v, e_a)
 
     attainable = copy_bandwidth(torch, mib=max(a.calibration_copy_mib, 1024), reps=5)
     if a.calibration_copy_mib > 0:       # one more copy of exactly the stated size, for the profiler
@@ -755,7 +759,7 @@ def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
             bin_t.append(e0.elapsed_time(mid))
             tile_t.append(mid.elapsed_time(e1))
         bin_ms, tile_ms = sum(bin_t) / len(bin_t), sum(tile_t) / len(tile_t)
-        kernels["backward_tile"] = entry("tile_backward_kernel (all gradients, one launch)", tile_ms, min(tile_t), bwd_bytes,
+        kernels["backward_tile"] = entry("tile kernel of the binned backward (all gradients, one launch)", tile_ms, min(tile_t), bwd_bytes,
                                          "backward_tile")
         kernels["backward_binning"] = {"kernel": "plan_and_clear + bin_count + bin_scan (whose further blocks clear gradient rows) + bin_fill_sorted (+ their plain forms, which step aside)",
                                        "avg_ms": round(bin_ms, 4), "min_ms": round(min(bin_t), 4)}
@@ -774,7 +778,7 @@ def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if bf16 else "f32", "data": "synthetic",
+        "dtype": "bf16" if bf16 else "f64" if f64 else "f32", "data": "synthetic",
         "config": {"workload": f"{a.workload}: B={w.B} Q={w.Q} M={w.M} C={w.C} L={w.L} "
                                f"levels={'/'.join(f'{h}x{x}' for h, x in w.levels)} D={w.D} P={w.P} "
                                f"({w.points} sampled points), one-stage Function forward+backward",
@@ -789,7 +793,7 @@ def run(a, torch, _ext, _lib, L_, F1, WORKLOADS, make_inputs, user_options):
         "roofline": roofline,
         "roofline_whole_backward": whole_bwd,
     }
-    if a.variants:
+    if a.variants and not f64:
         result["variants"] = variant_timings(_ext, torch, vd, dd, shapes, lsi, ld, ad, go, max(a.kernel_reps // 2, 3))
     if a.cpu_seconds > 0:
         result["cpu_baseline"] = cpu_baseline(w, a.cpu_seconds)
