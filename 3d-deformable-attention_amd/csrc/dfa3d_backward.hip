@@ -361,7 +361,7 @@ static hipError_t launch_bwd_cfg(const BwdArgs &a, hipStream_t stream) {
 
 template <typename T, typename A>
 static hipError_t launch_bwd_typed(const BwdArgs &a, hipStream_t stream) {
-  const RowTiling rt = pick_row_tiling(a.C, (int)sizeof(T), a.vec_hint);
+  const RowTiling rt = pick_row_tiling(a.C, (int)sizeof(T), a.vec_hint, true);
 #define DFA3D_CASE(V, R) \
   if (rt.vec == V && rt.lpr == R) return launch_bwd_cfg<T, A, V, R>(a, stream);
   DFA3D_ROW_TILINGS(DFA3D_CASE)

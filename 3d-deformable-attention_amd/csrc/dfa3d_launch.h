@@ -21,10 +21,13 @@ inline bool tiling_exists(int vec, int lpr) {
 }
 
 // vec_hint > 0 forces that vector width when it fits the channel count.
-inline RowTiling pick_row_tiling(int C, int elem_size, int vec_hint) {
-  // widest vectors first: 16 bytes per lane (fp32) measured fastest for the row gathers
-  const int order_wide[3] = {4, 2, 1}, order_f64[3] = {2, 4, 1};
-  const int *order = elem_size <= 4 ? order_wide : order_f64;
+inline RowTiling pick_row_tiling(int C, int elem_size, int vec_hint, bool atomics = false) {
+  // Gathers: widest vectors first, 16 bytes per lane (fp32) measured fastest.  Rows added with device-memory atomics
+  // (one instruction per channel of a lane, each touching every row of the wavefront again): narrowest first, the
+  // memory side retires cache-line requests, not bytes (base shape: 11.6 / 17.5 / 29.8 ms for 1 / 2 / 4 channels per
+  // lane in float, 15.9 / 26.8 / 49.6 ms in double).
+  const int order_wide[3] = {4, 2, 1}, order_f64[3] = {2, 4, 1}, order_atomics[3] = {1, 2, 4};
+  const int *order = atomics ? order_atomics : elem_size <= 4 ? order_wide : order_f64;
   for (int i = -1; i < 3; ++i) {
     const int vec = i < 0 ? vec_hint : order[i];
     if (vec != 1 && vec != 2 && vec != 4) continue;

@@ -259,13 +259,28 @@ def summarize_json(path):
     return out
 
 
+def source_stamp():
+    """What the measured library was built from: the digest of the HIP sources (the same one bench.py checks the
+    traffic figures against) and, where git is at hand, the commit with a mark for uncommitted changes."""
+    import subprocess
+    stamp = f"kernel sources sha256 {sources_digest()[:16]}"
+    try:
+        head = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True, check=True).stdout.strip()
+        dirty = subprocess.run(["git", "-C", ROOT, "status", "--porcelain", "--", "3d-deformable-attention_amd", "bench.py"],
+                               capture_output=True, text=True, check=True).stdout.strip()
+        stamp += f", git {head}" + (" + uncommitted changes" if dirty else "")
+    except (OSError, subprocess.CalledProcessError):
+        pass
+    return stamp
+
+
 def summarize(name, dirs, commands):
     """Per-kernel tables from rocprofv3's rocpd databases (kernel durations; counters per dispatch, averaged) as
     text under profiles/, and the HBM-side bytes of the operator's kernels (FETCH_SIZE / WRITE_SIZE, each scaled
     by what the same counter reads for the yardstick copy of known size in the same run) into
     profiles/hbm_traffic.json."""
     import sqlite3
-    lines = [f"# {c}" for c in commands]
+    lines = [f"# {c}" for c in commands] + [f"# {source_stamp()}"]
     scale, raw, workload = {}, {}, None
     for path in [d for d in dirs if d.endswith(".json")]:
         lines += summarize_json(path)
