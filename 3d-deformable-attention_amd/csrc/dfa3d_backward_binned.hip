@@ -435,23 +435,32 @@ __device__ __forceinline__ void clear_unstored(const BinWorkspace &ws, const Cle
   }
 }
 
-// Block 0 scans; further blocks, if any, clear the gradient rows that need it meanwhile (both only read the
-// counts: the scan is one workgroup's work and would leave the rest of the GPU idle).
-__global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws, ClearArgs ca) {
-  if (blockIdx.x > 0) {
-    clear_unstored(ws, ca, blockIdx.x - 1, gridDim.x - 1);
+// The first `scan_blocks` blocks scan, 4096 bins each (four consecutive bins per thread; their loads are independent,
+// so a round costs one memory latency), in turns if there are more bins than that.  A block needs no word from the
+// blocks before it: it adds up the counts of all bins before its own (a few dozen loads per thread for tens of
+// thousands of bins), which is cheaper than one workgroup walking all bins and writing every work item from one CU.
+// Further blocks, if any, clear the gradient rows that need it meanwhile (both kinds only read the counts).
+__global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws, ClearArgs ca, int scan_blocks) {
+  if ((int)blockIdx.x >= scan_blocks) {
+    clear_unstored(ws, ca, blockIdx.x - scan_blocks, gridDim.x - scan_blocks);
     return;
   }
-
-  // One workgroup walks the bins 4096 at a time: four consecutive bins per thread (their loads are
-  // independent, so a round costs one memory latency), a workgroup-wide exclusive scan of points and of
-  // work items, and a running carry.
-  __shared__ int s_pts[16], s_chk[16], s_carry[2];
+  __shared__ int s_pts[16], s_chk[16], s_bp[16], s_bc[16];
   const int n = ws.plan->total_bins, ch = ws.plan->chunk, per_class = ws.plan->bins_per_class;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  if (threadIdx.x == 0) { s_carry[0] = 0; s_carry[1] = 0; }
-  __syncthreads();
-  for (int base = 0; base < n; base += 4096) {
+  for (int base = (int)blockIdx.x * 4096; base < n; base += scan_blocks * 4096) {
+    // points and work items of the bins before this block's: every thread its share, summed over the wavefront
+    int bp = 0, bc = 0;
+    for (int i = threadIdx.x; i < base; i += 1024) {
+      const int c = ws.counts[i];
+      bp += c;
+      bc += (c + ch - 1) / ch;
+    }
+#pragma unroll
+    for (int off = kWave / 2; off >= 1; off >>= 1) {
+      bp += __shfl_xor(bp, off, kWave);
+      bc += __shfl_xor(bc, off, kWave);
+    }
     const int i0 = base + (int)threadIdx.x * 4;
     int c[4], k[4];
 #pragma unroll
@@ -466,10 +475,15 @@ __global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws, ClearAr
       const int up = __shfl_up(ip, off, kWave), uc = __shfl_up(ic, off, kWave);
       if (lane >= off) { ip += up; ic += uc; }
     }
+    __syncthreads();                                         // the tables of the turn before have been read
     if (lane == kWave - 1) { s_pts[wave] = ip; s_chk[wave] = ic; }
+    if (lane == 0) { s_bp[wave] = bp; s_bc[wave] = bc; }
     __syncthreads();
-    int run_p = s_carry[0] + ip - pts, run_c = s_carry[1] + ic - chk;
-    for (int w = 0; w < wave; ++w) { run_p += s_pts[w]; run_c += s_chk[w]; }
+    int run_p = ip - pts, run_c = ic - chk;
+    for (int w = 0; w < 16; ++w) {
+      run_p += s_bp[w] + (w < wave ? s_pts[w] : 0);
+      run_c += s_bc[w] + (w < wave ? s_chk[w] : 0);
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int i = i0 + j;
@@ -480,15 +494,12 @@ __global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws, ClearAr
           ws.items[run_c + t] = make_int4(i, run_p + t * ch, min(ch, c[j] - t * ch), k[j]);
         run_p += c[j];
         run_c += k[j];
+        if (i == n - 1) {
+          ws.plan->total_chunks = run_c;
+          ws.plan->class_start[kClasses] = run_c;
+        }
       }
     }
-    __syncthreads();                                         // everyone has read the carry and the wave sums
-    if (threadIdx.x == 1023) { s_carry[0] = run_p; s_carry[1] = run_c; }
-    __syncthreads();
-  }
-  if (threadIdx.x == 0) {
-    ws.plan->total_chunks = s_carry[1];
-    ws.plan->class_start[kClasses] = s_carry[1];
   }
 }
 
@@ -1476,7 +1487,10 @@ static hipError_t run_binning(const BwdArgs &a, const BinWorkspace &ws, int ty, 
     const size_t rows = (size_t)a.B * a.S * a.M;
     clear_blocks = (unsigned)((rows + 1023) / 1024 < 4096 ? (rows + 1023) / 1024 : 4096);
   }
-  hipLaunchKernelGGL(bin_scan_kernel, dim3(1 + clear_blocks), dim3(1024), 0, stream, ws, ca);
+  // scanning blocks for the most bins there can be (the plan kernel knows how many there are), 64 at most
+  const size_t max_bins = (size_t)mb * slot_count(a.B, a.M);
+  const unsigned scan_blocks = (unsigned)(max_bins + 4095) / 4096 < 64 ? (unsigned)((max_bins + 4095) / 4096) : 64u;
+  hipLaunchKernelGGL(bin_scan_kernel, dim3(scan_blocks + clear_blocks), dim3(1024), 0, stream, ws, ca, (int)scan_blocks);
   if (LP <= kStage) {
     if (hipError_t e = allow_lds(bin_fill_sorted_kernel, kSortedFillLds)) return e;
     hipLaunchKernelGGL(bin_fill_sorted_kernel, dim3((unsigned)blocks2), dim3(kFillThreads), kSortedFillLds, stream, ws, (const float *)a.loc,

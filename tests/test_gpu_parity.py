@@ -586,7 +586,8 @@ def test_fp32_random_shapes_two_stage_and_shared_distribution(oracle, seed):
 
 @pytest.mark.parametrize("setting", [dict(block=256), dict(**{"pass": 128}), dict(**{"pass": 64}), dict(tile=404),
                                      dict(tile=816), dict(tile=203, chunk=64), dict(chunk=256), dict(vec=4),
-                                     dict(vec=8, tile=404), dict(iters=3)],
+                                     dict(vec=8, tile=404), dict(iters=3), dict(tile=608), dict(tile=408, chunk=100),
+                                     dict(tile=202), dict(tile=101, chunk=64)],
                          ids=lambda d: "-".join(f"{k}{v}" for k, v in d.items()))
 def test_launch_options_do_not_change_results(oracle, setting):
     """Tile shape, workgroup size, points per pass, points per work item and channels per lane of the binned
