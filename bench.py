@@ -450,6 +450,33 @@ def event_time(fn, reps, prep=None):
     return total / reps, best
 
 
+def torch_volume_form_ms(torch, inp, levels, reps=10):
+    """Forward of the operator on the CPU with torch.nn.functional.grid_sample on the 5-D volume
+    V[c, d, h, w] = value[h, w, c] * dist[h, w, d] (align_corners=False, zero padding), per level."""
+    import torch.nn.functional as F
+    value, dist, loc, attn = inp["value"], inp["value_dpt_dist"], inp["sampling_locations"], inp["attention_weights"]
+    B, S, M, C = value.shape
+    D, Q, P = dist.shape[-1], loc.shape[1], loc.shape[4]
+
+    def run():
+        out, start = value.new_zeros(B * M, C, Q), 0
+        for l, (H, W) in enumerate(levels):
+            v = value[:, start:start + H * W].reshape(B, H, W, M, C).permute(0, 3, 4, 1, 2).reshape(B * M, C, 1, H, W)
+            d = dist[:, start:start + H * W].reshape(B, H, W, M, D).permute(0, 3, 4, 1, 2).reshape(B * M, 1, D, H, W)
+            start += H * W
+            grid = (2 * loc[:, :, :, l] - 1).permute(0, 2, 1, 3, 4).reshape(B * M, Q, P, 1, 3)
+            s = F.grid_sample(v * d, grid, mode="bilinear", padding_mode="zeros", align_corners=False)
+            out = out + (s.squeeze(-1) * attn[:, :, :, l].permute(0, 2, 1, 3).reshape(B * M, 1, Q, P)).sum(-1)
+        return out
+
+    with torch.no_grad():
+        run()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            run()
+    return (time.perf_counter() - t0) * 1e3 / reps
+
+
 def cpu_baseline(w, budget_s):
     """Forward+backward of the C restatement on a bounded sample (fewer queries, same everything else)."""
     import torch
@@ -480,8 +507,13 @@ def cpu_baseline(w, budget_s):
     for _ in range(50):
         orc.dfa3d_forward(*uargs)
     unit_ms = (time.perf_counter() - t0) * 1e3 / 50
+    # and the same configuration as a user without any extension would run it on these cores: the operator as
+    # PyTorch's own trilinear grid_sample of the expanded volume value (x) dist (the equivalence the reference's
+    # README.md:18 states), forward only
+    torch_ms = torch_volume_form_ms(torch, unit, WORKLOADS["unit"].levels)
     return {"value": sample.points / per_step, "unit": "points/s", "cores": threads, "kind": "port",
             "unit_workload_forward_ms": round(unit_ms, 4),
+            "unit_workload_forward_torch_grid_sample_ms": round(torch_ms, 4),
             "unit_workload_forward_points_per_s": WORKLOADS["unit"].points / (unit_ms * 1e-3),
             "sample": f"{w.name} workload with Q={sample.Q} of {w.Q} queries per batch element "
                       f"({sample.points} points), forward+backward, {reps} repetition(s), {per_step * 1e3:.1f} ms each; "
