@@ -435,12 +435,15 @@ __device__ __forceinline__ void clear_unstored(const BinWorkspace &ws, const Cle
   }
 }
 
-// The first `scan_blocks` blocks scan, 4096 bins each (four consecutive bins per thread; their loads are independent,
-// so a round costs one memory latency), in turns if there are more bins than that.  A block needs no word from the
-// blocks before it: it adds up the counts of all bins before its own (a few dozen loads per thread for tens of
-// thousands of bins), which is cheaper than one workgroup walking all bins and writing every work item from one CU.
-// Further blocks, if any, clear the gradient rows that need it meanwhile (both kinds only read the counts).
-__global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws, ClearArgs ca, int scan_blocks) {
+// work items of a bin with c points (most bins fit one item, which saves the division)
+__device__ __forceinline__ int items_of_bin(int c, int ch) { return c <= ch ? (c > 0 ? 1 : 0) : (c + ch - 1) / ch; }
+
+// The first `scan_blocks` blocks scan, 1024 bins each (in turns if there are more bins than that).  A block needs no
+// word from the blocks before it: it adds up the counts of all bins before its own (a few dozen loads per thread for
+// tens of thousands of bins), which is cheaper than one workgroup walking all bins and writing every work item from
+// one CU.  Further blocks, if any, clear the gradient rows that need it meanwhile (both kinds only read the counts);
+// the kernel is held to 64 registers so that two such workgroups fit a CU.
+__global__ __launch_bounds__(1024, 8) void bin_scan_kernel(BinWorkspace ws, ClearArgs ca, int scan_blocks) {
   if ((int)blockIdx.x >= scan_blocks) {
     clear_unstored(ws, ca, blockIdx.x - scan_blocks, gridDim.x - scan_blocks);
     return;
@@ -448,56 +451,37 @@ __global__ __launch_bounds__(1024) void bin_scan_kernel(BinWorkspace ws, ClearAr
   __shared__ int s_pts[16], s_chk[16], s_bp[16], s_bc[16];
   const int n = ws.plan->total_bins, ch = ws.plan->chunk, per_class = ws.plan->bins_per_class;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  for (int base = (int)blockIdx.x * 4096; base < n; base += scan_blocks * 4096) {
+  for (int base = (int)blockIdx.x * 1024; base < n; base += scan_blocks * 1024) {
     // points and work items of the bins before this block's: every thread its share, summed over the wavefront
     int bp = 0, bc = 0;
+#pragma unroll 4
     for (int i = threadIdx.x; i < base; i += 1024) {
       const int c = ws.counts[i];
       bp += c;
-      bc += (c + ch - 1) / ch;
+      bc += items_of_bin(c, ch);
     }
-#pragma unroll
-    for (int off = kWave / 2; off >= 1; off >>= 1) {
-      bp += __shfl_xor(bp, off, kWave);
-      bc += __shfl_xor(bc, off, kWave);
-    }
-    const int i0 = base + (int)threadIdx.x * 4;
-    int c[4], k[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      c[j] = i0 + j < n ? ws.counts[i0 + j] : 0;
-      k[j] = (c[j] + ch - 1) / ch;
-    }
-    const int pts = c[0] + c[1] + c[2] + c[3], chk = k[0] + k[1] + k[2] + k[3];
-    int ip = pts, ic = chk;                                  // inclusive scans within the wavefront
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-      const int up = __shfl_up(ip, off, kWave), uc = __shfl_up(ic, off, kWave);
-      if (lane >= off) { ip += up; ic += uc; }
-    }
+    bp = __builtin_amdgcn_readlane(wave_inclusive_scan(bp), kWave - 1);
+    bc = __builtin_amdgcn_readlane(wave_inclusive_scan(bc), kWave - 1);
+    const int i = base + (int)threadIdx.x;
+    const int c = i < n ? ws.counts[i] : 0, k = items_of_bin(c, ch);
+    const int ip = wave_inclusive_scan(c), ic = wave_inclusive_scan(k);      // inclusive scans within the wavefront
     __syncthreads();                                         // the tables of the turn before have been read
     if (lane == kWave - 1) { s_pts[wave] = ip; s_chk[wave] = ic; }
     if (lane == 0) { s_bp[wave] = bp; s_bc[wave] = bc; }
     __syncthreads();
-    int run_p = ip - pts, run_c = ic - chk;
+    int run_p = ip - c, run_c = ic - k;
     for (int w = 0; w < 16; ++w) {
       run_p += s_bp[w] + (w < wave ? s_pts[w] : 0);
       run_c += s_bc[w] + (w < wave ? s_chk[w] : 0);
     }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int i = i0 + j;
-      if (i < n) {
-        if (i % per_class == 0) ws.plan->class_start[i / per_class] = run_c;
-        ws.cursor[i] = run_p;
-        for (int t = 0; t < k[j]; ++t)
-          ws.items[run_c + t] = make_int4(i, run_p + t * ch, min(ch, c[j] - t * ch), k[j]);
-        run_p += c[j];
-        run_c += k[j];
-        if (i == n - 1) {
-          ws.plan->total_chunks = run_c;
-          ws.plan->class_start[kClasses] = run_c;
-        }
+    if (i < n) {
+      if (i % per_class == 0) ws.plan->class_start[i / per_class] = run_c;
+      ws.cursor[i] = run_p;
+      for (int t = 0; t < k; ++t)
+        ws.items[run_c + t] = make_int4(i, run_p + t * ch, min(ch, c - t * ch), k);
+      if (i == n - 1) {
+        ws.plan->total_chunks = run_c + k;
+        ws.plan->class_start[kClasses] = run_c + k;
       }
     }
   }
@@ -1489,7 +1473,7 @@ static hipError_t run_binning(const BwdArgs &a, const BinWorkspace &ws, int ty, 
   }
   // scanning blocks for the most bins there can be (the plan kernel knows how many there are), 64 at most
   const size_t max_bins = (size_t)mb * slot_count(a.B, a.M);
-  const unsigned scan_blocks = (unsigned)(max_bins + 4095) / 4096 < 64 ? (unsigned)((max_bins + 4095) / 4096) : 64u;
+  const unsigned scan_blocks = (max_bins + 1023) / 1024 < 64 ? (unsigned)((max_bins + 1023) / 1024) : 64u;
   hipLaunchKernelGGL(bin_scan_kernel, dim3(scan_blocks + clear_blocks), dim3(1024), 0, stream, ws, ca, (int)scan_blocks);
   if (LP <= kStage) {
     if (hipError_t e = allow_lds(bin_fill_sorted_kernel, kSortedFillLds)) return e;
