@@ -93,15 +93,20 @@ WORKLOADS = {
     # alone, whose value rows and distributions of one (batch, head) fit an XCD's L2 (2.9 MB).  base_band: all four
     # levels, but the locations of level 0 confined to the upper third of the map, i.e. what a forward that walks
     # level 0 band by band would find in the L2 during one band.
+    # base_fine / base_fine_band: level 0 alone (3.84 M points; the tile kernel's work items then all take a single
+    # pass), and with its locations confined to that band.
     "base_coarse": Workload("base_coarse", B=6, Q=10000, levels=_BASE_LEVELS[1:], D=64, P=8, depth_sigma=2.0),
     "base_band": Workload("base_band", B=6, Q=10000, levels=_BASE_LEVELS, D=64, P=8, depth_sigma=2.0, loc="band"),
+    "base_fine": Workload("base_fine", B=6, Q=10000, levels=_BASE_LEVELS[:1], D=64, P=8, depth_sigma=2.0),
+    "base_fine_band": Workload("base_fine_band", B=6, Q=10000, levels=_BASE_LEVELS[:1], D=64, P=8, depth_sigma=2.0,
+                               loc="band"),
     # dense BEV grid, clustered locations
     "dense": Workload("dense", B=6, Q=40000, levels=_BASE_LEVELS, D=128, P=8, loc="normal",
                       loc_lo=-0.1, loc_hi=1.1, depth_sigma=2.0),
 }
 
 SEEDS = {"unit": 1, "small": 2, "base": 3, "base_peaky": 4, "dense": 5, "unittest": 6, "base_coherent": 7,
-         "base_coarse": 3, "base_band": 3}
+         "base_coarse": 3, "base_band": 3, "base_fine": 3, "base_fine_band": 3}
 
 
 def scaled(w: Workload, B=None, Q=None, name=None) -> Workload:
