@@ -64,7 +64,7 @@ __host__ __device__ inline CellLds cell_lds_layout(int ty, int tx, int D) {
   const int stage_words = (kCellPass + 1) * kGPitch, acc_words = kCellMax * 4 * kCellC;
   o.sw = o.gstage + (stage_words > acc_words ? stage_words : acc_words);
   o.sslot = o.sw + kCellPass * 4;
-  o.dots = o.sslot + kCellPass;
+  o.dots = o.sslot + kCellPass / 2;                          // 16-bit point slots
   o.cnt = o.dots + kCellPass * 4 + kWave;                    // + one scrap word per lane
   o.offs = o.cnt + 2 * kCellMax;
   o.goff = o.offs + kCellMax + 1;
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(kCellBlock, 4) void cell_backward_kernel(
   float *gd = smem + lay.gd, *gstage = smem + lay.gstage, *dots = smem + lay.dots;
   uint32_t *bitmap = reinterpret_cast<uint32_t *>(smem + lay.bits);
   float4 *s_w = reinterpret_cast<float4 *>(smem + lay.sw);
-  int *s_slot = reinterpret_cast<int *>(smem + lay.sslot);
+  uint16_t *s_slot = reinterpret_cast<uint16_t *>(smem + lay.sslot);
   int *cnt = reinterpret_cast<int *>(smem + lay.cnt), *offs = reinterpret_cast<int *>(smem + lay.offs);
   uint32_t *goff = reinterpret_cast<uint32_t *>(smem + lay.goff);
   const int cl = lane % LPR;
@@ -524,7 +524,7 @@ const ItemGeom q = uniform(s_geom[which]);
           if (lane == kWave - 1) offs[kCellMax] = inc;
           if (my_cell >= 0) {
             const int pos = offs[my_cell] + my_rank;
-            s_slot[pos] = pslot;
+            s_slot[pos] = (uint16_t)pslot;
             s_w[pos] = pw;
           }
         }
