@@ -1255,9 +1255,9 @@ static TileConfig pick_tile_config(int kind, int C, int D, int tile_hint, int bl
     // room for two workgroups per CU, else for one.
     static const int order[][2] = {{8, 8}, {6, 8}, {4, 8}, {4, 4}, {2, 4}, {2, 2}, {1, 1}};
     const int hy = tile_hint / 100, hx = tile_hint % 100;
-    // two workgroups per CU: half of the 160 KB less the kernel's static 448 bytes (a depth tile of 112 bins on 8x8
-    // pixels just fits)
-    for (size_t budget : {(size_t)80 * 1024 - 512, (size_t)150 * 1024}) {
+    // two workgroups per CU: half of the 160 KB less the kernel's static LDS (a depth tile of 112 bins on 8x8 pixels
+    // just fits; 128 bins would fit on 8x7 pixels, which is no faster than 6x8 on the dense workload: 5.66 against 5.65 ms)
+    for (size_t budget : {cell_kernel_half_cu_lds(), (size_t)150 * 1024}) {
       for (auto &t : order) {
         const int ty = tile_hint > 0 ? hy : t[0], tx = tile_hint > 0 ? hx : t[1];
         const int Dk = kind == 1 ? 0 : D;

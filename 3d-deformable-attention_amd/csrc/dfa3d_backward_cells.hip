@@ -65,7 +65,7 @@ __host__ __device__ inline CellLds cell_lds_layout(int ty, int tx, int D) {
   o.sw = o.gstage + (stage_words > acc_words ? stage_words : acc_words);
   o.sslot = o.sw + kCellPass * 4;
   o.dots = o.sslot + kCellPass / 2;                          // 16-bit point slots
-  o.cnt = o.dots + kCellPass * 4 + kWave;                    // + one scrap word per lane
+  o.cnt = o.dots + kCellPass * 4;
   o.offs = o.cnt + 2 * kCellMax;
   o.goff = o.offs + kCellMax + 1;
   o.total = o.goff + kCellPass;
@@ -110,6 +110,10 @@ struct CellFetch {
 };
 // a work item, decoded
 struct ItemGeom { int bin, seg, n_item, chunks, b, m, H, W, Dd, start, y0, x0; };
+// what the kernel declares as static LDS (level tables, the fetching thread's state, three item records): the dynamic
+// block of each of two workgroups on a CU may be half of the CU's 160 KB less this
+constexpr size_t kCellStaticLds = 4 * DFA3D_MAX_LEVELS * sizeof(int) + sizeof(CellFetch) + 3 * sizeof(ItemGeom);
+size_t cell_kernel_half_cu_lds() { return 80 * 1024 - kCellStaticLds; }
 // an item record read from LDS is the same in every lane: keep it in scalar registers
 __device__ __forceinline__ ItemGeom uniform(const ItemGeom &g) {
   ItemGeom u;

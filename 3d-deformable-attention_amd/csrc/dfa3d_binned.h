@@ -188,6 +188,7 @@ template <int VEC> __device__ __forceinline__ void lds_ld(const float *p, float 
 // The cell-owned tile kernel (dfa3d_backward_cells.hip): rows of 32 channels, tiles of at most 64 pixels.
 bool cell_kernel_applies(int C, int D, int ty, int tx, bool fused);
 size_t cell_kernel_lds_bytes(int ty, int tx, int D);
+size_t cell_kernel_half_cu_lds();      // the most dynamic LDS with which two of its workgroups fit a CU
 const void *cell_kernel_symbol(int dtype, bool fused);
 hipError_t launch_cell_kernel(const BwdArgs &a, int dtype, const BinWorkspace &ws, size_t lds, int grid, float *gd_heads,
                               hipStream_t stream);
